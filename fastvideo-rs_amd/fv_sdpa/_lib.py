@@ -1,0 +1,76 @@
+"""Loader for libfv_sdpa_hip.so (the C ABI in include/fv_sdpa_hip.h).
+
+There is no fallback: a missing library or symbol raises, and no function here
+ever computes on the host.
+"""
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG, "libfv_sdpa_hip.so")
+CSRC = os.path.join(_PKG, "csrc")
+
+FV_OK = 0
+FV_DECLINED = 1
+
+_sz = C.c_size_t
+_vp = C.c_void_p
+
+# name -> (restype, argtypes); must list every symbol include/fv_sdpa_hip.h declares
+SIGNATURES = {
+    "fv_sdpa_last_error": (C.c_char_p, []),
+    "fv_sdpa_arch": (C.c_char_p, []),
+    "fv_sdpa_supported": (C.c_int, [_sz, _sz, _sz, _sz, _sz]),
+    "fv_sdpa_dense_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float, _vp]),
+    "fv_sdpa_block_causal_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float,
+                                            _sz, _sz, _sz, _vp]),
+    "fv_cast_f32_bf16": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "fv_cast_bf16_f32": (C.c_int, [_vp, _vp, _sz, _vp]),
+}
+
+_lib = None
+
+
+class FvError(RuntimeError):
+    """A negative return of the C ABI (a HIP error)."""
+
+
+class FvDeclined(RuntimeError):
+    """FV_DECLINED: the kernel does not take this call; nothing ran."""
+
+
+def build(force=True):
+    """Compile the library in-tree with the committed Makefile (hipcc, gfx950)."""
+    import subprocess
+
+    cmd = ["make", "-C", CSRC, "-j8"] + (["-B"] if force else [])
+    subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(there is no CPU fallback)")
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)  # AttributeError if the symbol is missing
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def last_error():
+    return lib().fv_sdpa_last_error().decode()
+
+
+def check(rc):
+    if rc == FV_OK:
+        return
+    if rc == FV_DECLINED:
+        raise FvDeclined(last_error())
+    raise FvError(f"rc={rc}: {last_error()}")

@@ -1,0 +1,69 @@
+"""torch-tensor wrappers over the kernel-level C ABI (include/fv_sdpa_hip.h).
+
+Every wrapper validates on the host what the kernel assumes (device, dtype,
+contiguity, shapes) before the launch.
+"""
+import math
+
+import torch
+
+from . import _lib
+
+__all__ = ["sdpa_dense_bf16", "sdpa_block_causal_bf16", "cast_f32_bf16", "cast_bf16_f32", "sdpa_supported"]
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(t, dtype, name):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous()):
+        raise ValueError(f"{name}: want a contiguous CUDA tensor of {dtype}")
+
+
+def _bhsd(q, k, v):
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        _need(t, torch.bfloat16, n)
+    if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise ValueError("want [bh, s, d] operands")
+    bh, sq, d = q.shape
+    if k.shape != v.shape or k.shape[0] != bh or k.shape[2] != d:
+        raise ValueError(f"k/v {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
+    return bh, sq, k.shape[1], d
+
+
+def sdpa_supported(b, h, sq, sk, d):
+    return bool(_lib.lib().fv_sdpa_supported(b, h, sq, sk, d))
+
+
+def sdpa_dense_bf16(q, k, v, scale=None, out_bf16=False):
+    bh, sq, sk, d = _bhsd(q, k, v)
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    out = torch.empty((bh, sq, d), device=q.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    _lib.check(_lib.lib().fv_sdpa_dense_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                             int(out_bf16), bh, sq, sk, d, scale, _stream()))
+    return out
+
+
+def sdpa_block_causal_bf16(q, k, v, block_tokens, window=0, sink=0, scale=None, out_bf16=False):
+    bh, sq, sk, d = _bhsd(q, k, v)
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    out = torch.empty((bh, sq, d), device=q.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    _lib.check(_lib.lib().fv_sdpa_block_causal_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                                    int(out_bf16), bh, sq, sk, d, scale, block_tokens, window,
+                                                    sink, _stream()))
+    return out
+
+
+def cast_f32_bf16(x):
+    _need(x, torch.float32, "x")
+    y = torch.empty(x.shape, device=x.device, dtype=torch.bfloat16)
+    _lib.check(_lib.lib().fv_cast_f32_bf16(x.data_ptr(), y.data_ptr(), x.numel(), _stream()))
+    return y
+
+
+def cast_bf16_f32(x):
+    _need(x, torch.bfloat16, "x")
+    y = torch.empty(x.shape, device=x.device, dtype=torch.float32)
+    _lib.check(_lib.lib().fv_cast_bf16_f32(x.data_ptr(), y.data_ptr(), x.numel(), _stream()))
+    return y

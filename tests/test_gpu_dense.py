@@ -1,0 +1,143 @@
+"""Parity of the gfx950 dense flash kernel (through the C ABI) against the CPU
+oracle's fp32 composed SDPA. Shapes follow the reference's flash_mma table
+(crates/fastvideo-gpucheck/src/kernels.rs:2286-2297, d = 128 rows) plus the
+BASELINE configs; tolerances: max|delta| <= 1e-2, cosine >= 0.9999 vs the fp32
+oracle on identical bf16-valued inputs, rel_l2 <= 1e-2 vs the oracle on the
+unrounded inputs, <= 2e-3 on rounded inputs (kernels.rs:2314-2328).
+"""
+import numpy as np
+import pytest
+
+from util import announce, assert_parity, metrics, qkv, randn, sample_rows, to_dev_bf16
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [  # (bh, sq, sk, std)
+    (1, 1, 1, 1.0),
+    (2, 64, 64, 1.0),
+    (6, 257, 257, 1.0),
+    (4, 300, 512, 1.0),
+    (3, 130, 1, 1.0),
+    (2, 63, 4097, 1.0),
+    (4, 1024, 1024, 2.0),
+    (2, 2048, 2048, 1.0),
+    (12, 320, 320, 1.0),   # BASELINE config 1
+    (2, 128, 64, 1.0),
+    (1, 129, 65, 1.0),
+    (1, 127, 63, 1.0),
+]
+
+
+@pytest.fixture(scope="module")
+def fv():
+    import torch
+
+    assert torch.cuda.is_available()
+    import fv_sdpa
+
+    fv_sdpa.lib()
+    return fv_sdpa
+
+
+@pytest.mark.parametrize("bh,sq,sk,std", SHAPES)
+def test_dense_matches_composed_oracle(fv, oracle, bh, sq, sk, std):
+    import torch
+
+    d, seed = 128, 1000 + bh * 7 + sq
+    announce(f"dense bh={bh} sq={sq} sk={sk} d={d} std={std} seed={seed}")
+    q, k, v = qkv(seed, bh, sq, sk, d, std)
+    want = oracle.sdpa_composed(q, k, v)
+    qd, kd, vd = (to_dev_bf16(x) for x in (q, k, v))
+    got = fv.sdpa_dense_bf16(qd, kd, vd, out_bf16=False)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    m = assert_parity(got, want, f"dense_{bh}x{sq}x{sk}_s{std}", max_abs=1e-2 if std == 1.0 else 5e-2)
+    assert m["rel_l2"] <= 2e-3 * (1 if std == 1.0 else 3)
+    got16 = fv.sdpa_dense_bf16(qd, kd, vd, out_bf16=True)
+    torch.cuda.synchronize()
+    got16 = got16.float().cpu().numpy()
+    assert_parity(got16, want, f"dense_{bh}x{sq}x{sk}_bf16out", max_abs=2e-2 if std == 1.0 else 6e-2)
+    assert metrics(got16, want)["rel_l2"] <= 1e-2
+    # bf16 out is the RNE rounding of the f32 out
+    assert np.array_equal(got16, oracle.quantize_bf16(got))
+
+
+def test_dense_vs_unrounded_f32_inputs(fv, oracle):
+    import torch
+
+    bh, sq, sk, d = 2, 512, 777, 128
+    announce(f"dense unrounded bh={bh} sq={sq} sk={sk}")
+    q, k, v = qkv(77, bh, sq, sk, d, round_bf16=False)
+    want = oracle.sdpa_composed(q, k, v)
+    got = fv.sdpa_dense_bf16(fv.cast_f32_bf16(torch.from_numpy(q).cuda()), fv.cast_f32_bf16(torch.from_numpy(k).cuda()),
+                             fv.cast_f32_bf16(torch.from_numpy(v).cuda()))
+    torch.cuda.synchronize()
+    m = metrics(got.cpu().numpy(), want)
+    print(m)
+    assert m["rel_l2"] <= 1e-2
+
+
+def test_scale_and_determinism(fv, oracle):
+    import torch
+
+    bh, sq, sk, d = 3, 200, 300, 128
+    announce("dense scale/determinism 3x200x300")
+    q, k, v = qkv(5, bh, sq, sk, d)
+    qd, kd, vd = (to_dev_bf16(x) for x in (q, k, v))
+    a = fv.sdpa_dense_bf16(qd, kd, vd, scale=0.05)
+    b = fv.sdpa_dense_bf16(qd, kd, vd, scale=0.05)
+    c = fv.sdpa_dense_bf16(qd, kd, vd)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert not torch.equal(a, c)
+    assert_parity(a.cpu().numpy(), oracle.sdpa_composed(q, k, v, scale=0.05), "dense_scale0.05")
+
+
+def test_large_scores_exercise_the_rescale(fv, oracle):
+    import torch
+
+    # keys ordered so the row max keeps growing: every tile forces a rescale
+    bh, sq, sk, d = 1, 128, 1024, 128
+    announce("dense growing-max 1x128x1024")
+    q, k, v = qkv(9, bh, sq, sk, d)
+    ramp = np.linspace(0.2, 3.0, sk, dtype=np.float32)[None, :, None]
+    k = oracle.quantize_bf16(np.abs(k) * ramp * np.sign(q.mean(axis=1, keepdims=True) + 1e-3))
+    want = oracle.sdpa_composed(q, k, v)
+    got = fv.sdpa_dense_bf16(*(to_dev_bf16(x) for x in (q, k, v)))
+    torch.cuda.synchronize()
+    assert_parity(got.cpu().numpy(), want, "dense_growing_max", max_abs=2e-2)
+
+
+def test_declines(fv):
+    import torch
+
+    x = torch.zeros((1, 4, 64), device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(fv.FvDeclined):
+        fv.sdpa_dense_bf16(x, x, x)          # d = 64: not built
+    y = torch.zeros((1, 4, 128), device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(fv.FvDeclined):
+        fv.sdpa_dense_bf16(y, y, y, scale=-1.0)
+    assert fv.sdpa_supported(1, 40, 38001, 38001, 128)
+    assert not fv.sdpa_supported(1, 8, 0, 1024, 128)
+    assert not fv.sdpa_supported(2, 40000, 64, 64, 128)
+
+
+def test_headline_shape_sampled_rows(fv, oracle):
+    """BASELINE config 2 at full size: S = 32760, H = 12; parity on sampled rows."""
+    import torch
+
+    bh, s, d = 12, 32760, 128
+    announce(f"dense headline bh={bh} s={s}")
+    g = torch.Generator(device="cuda").manual_seed(2024)
+    q, k, v = (torch.randn((bh, s, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    out = fv.sdpa_dense_bf16(q, k, v)
+    torch.cuda.synchronize()
+    rows = sample_rows(1, s, 48, extra=(0, 127, 128, s - 1, s - 57))
+    want = oracle.sdpa_composed_rows(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), rows)
+    assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, "dense_headline_rows")
+    # cross-attention: same queries against 512 keys
+    kc, vc = k[:, :512].contiguous(), v[:, :512].contiguous()
+    outc = fv.sdpa_dense_bf16(q, kc, vc)
+    torch.cuda.synchronize()
+    wantc = oracle.sdpa_composed_rows(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), rows)
+    assert_parity(outc[:, torch.from_numpy(rows).cuda()].cpu().numpy(), wantc, "cross_headline_rows")

@@ -1,0 +1,68 @@
+"""Shared helpers for the parity tests: seeded inputs and error metrics."""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "fastvideo-rs_amd")
+for p in (ROOT, PKG):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+# north-star tolerances: max|delta| <= 1e-2 and cosine >= 0.9999 against the
+# reference's fp32 host-math SDPA on identical seeded inputs
+MAX_ABS = 1e-2
+MIN_COS = 0.9999
+
+
+def randn(seed, shape, std=1.0):
+    """N(0, std) f32 from numpy's PCG64; tensors of one case use seed, seed+1, ..."""
+    return (np.random.Generator(np.random.PCG64(seed)).standard_normal(shape, dtype=np.float32) * np.float32(std))
+
+
+def qkv(seed, bh, sq, sk, d, std=1.0, round_bf16=True):
+    import oracle
+
+    q, k, v = randn(seed, (bh, sq, d), std), randn(seed + 1, (bh, sk, d), std), randn(seed + 2, (bh, sk, d))
+    if round_bf16:
+        q, k, v = (oracle.quantize_bf16(x) for x in (q, k, v))
+    return q, k, v
+
+
+def metrics(got, want):
+    got = np.asarray(got, dtype=np.float64).reshape(-1)
+    want = np.asarray(want, dtype=np.float64).reshape(-1)
+    diff = got - want
+    den = np.linalg.norm(want)
+    return {
+        "max_abs": float(np.abs(diff).max()) if diff.size else 0.0,
+        "rel_l2": float(np.linalg.norm(diff) / den) if den > 0 else float(np.linalg.norm(diff)),
+        "cosine": float(got @ want / (np.linalg.norm(got) * den)) if den > 0 and np.linalg.norm(got) > 0 else 1.0,
+    }
+
+
+def assert_parity(got, want, tag, max_abs=MAX_ABS, min_cos=MIN_COS):
+    assert np.isfinite(np.asarray(got)).all(), f"{tag}: non-finite output"
+    m = metrics(got, want)
+    print(f"[parity] {tag}: max_abs={m['max_abs']:.3e} rel_l2={m['rel_l2']:.3e} cos={m['cosine']:.7f}", flush=True)
+    assert m["max_abs"] <= max_abs, f"{tag}: max_abs {m['max_abs']} > {max_abs}"
+    assert m["cosine"] >= min_cos, f"{tag}: cosine {m['cosine']} < {min_cos}"
+    return m
+
+
+def announce(msg):
+    print(f"[gpu-case] {msg}", flush=True)
+
+
+def to_dev_bf16(x):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda().to(torch.bfloat16).contiguous()
+
+
+def sample_rows(seed, sq, n, extra=()):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    rows = set(int(r) for r in rng.choice(sq, size=min(n, sq), replace=False))
+    rows.update(int(r) for r in extra if 0 <= r < sq)
+    return np.array(sorted(rows), dtype=np.int64)
