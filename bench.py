@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Wan-1.3B 480p self-attention SDPA on one MI355X.
+
+One step = one call of the dense SDPA hot path (B=1, H=12, S=32760, d=128, bf16,
+scale 1/sqrt(128), non-causal) with Q/K/V already resident in HBM. Prints ONE
+JSON line: whole-call TFLOP/s (4*H*Sq*Sk*d FLOPs, the reference's convention,
+crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
+flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
+oracle timed on a bounded sample of query rows, extrapolated to the full call).
+
+Other workloads (--workload cross|causal|causal3|c5|tiny) are for the design notes;
+the driver's line is the default `self`.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "fastvideo-rs_amd"))
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (H, Sq, Sk, causal block_tokens or 0, description)
+    "self": (12, 32760, 32760, 0, "Wan2.1-1.3B 480x832x81 self-attention, B=1 H=12 S=32760 d=128 bf16 non-causal"),
+    "cross": (12, 32760, 512, 0, "Wan2.1-1.3B 480p text cross-attention, B=1 H=12 Sq=32760 Sk=512 d=128 bf16"),
+    "causal": (12, 32760, 32760, 1560, "Self-Forcing frame-causal, 21 frames x 1560 tokens, H=12 d=128 bf16"),
+    "causal3": (12, 32760, 32760, 4680, "Self-Forcing 3-frame blocks (reference geometry), H=12 d=128 bf16"),
+    "c5": (40, 75600, 75600, 0, "Wan2.1-14B 720p self-attention, B=1 H=40 S=75600 d=128 bf16"),
+    "c5cross": (40, 75600, 512, 0, "Wan2.1-14B 720p cross-attention, H=40 Sq=75600 Sk=512"),
+    "tiny": (12, 320, 320, 0, "tiny Wan-1.3B-shaped self-attention, H=12 S=320 d=128"),
+}
+
+
+def visible_pairs(sq, sk, bt):
+    if bt == 0:
+        return sq * sk
+    total = 0
+    for qb in range((sq + bt - 1) // bt):
+        nq = min(bt, sq - qb * bt)
+        total += nq * min(sk, (qb + 1) * bt)
+    return total
+
+
+def cpu_baseline(h, sq, sk, d, bt, flops_full, q, k, v, budget_s):
+    """Time the oracle's fp32 composed SDPA on a bounded sample of query rows."""
+    import numpy as np
+
+    import oracle
+
+    cores = os.cpu_count() or 1
+    threads = max(1, min(h, cores, 16))
+    qn, kn, vn = (x.float().cpu().numpy() for x in (q, k, v))
+    mask = (bt, 0, 0) if bt else None
+    rng = np.random.Generator(np.random.PCG64(7))
+
+    def run(n):
+        rows = np.sort(rng.choice(sq, size=min(n, sq), replace=False)).astype(np.int64)
+        t0 = time.perf_counter()
+        oracle.sdpa_composed_rows(qn, kn, vn, rows, mask_bc=mask, threads=threads)
+        return time.perf_counter() - t0, rows.size
+
+    t_probe, n_probe = run(min(16, sq))
+    per_row = max(t_probe / n_probe, 1e-9)
+    n = int(max(n_probe, min(sq, budget_s / per_row)))
+    t, n = run(n)
+    t_full = t * sq / n
+    return {
+        "value": flops_full / t_full / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{n} of {sq} query rows x all {h} heads x all {sk} keys in {t:.2f} s, "
+                  f"extrapolated x{sq / n:.1f} to {t_full:.1f} s/call; host has {cores} cores, "
+                  f"threads split heads only (as the reference's rayon matmul)",
+        "ms_per_call_extrapolated": t_full * 1e3,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
+    ap.add_argument("--out-bf16", type=int, default=1)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the full sequence on ONE GPU (no sharding, no collectives); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import fv_sdpa
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    fv_sdpa.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    h, sq, sk, bt, desc = WORKLOADS[args.workload]
+    d = 128
+    g = torch.Generator(device=dev).manual_seed(20240)
+    q = torch.randn((h, sq, d), generator=g, device=dev).to(torch.bfloat16)
+    k = torch.randn((h, sk, d), generator=g, device=dev).to(torch.bfloat16)
+    v = torch.randn((h, sk, d), generator=g, device=dev).to(torch.bfloat16)
+    out = torch.empty((h, sq, d), device=dev, dtype=torch.bfloat16 if args.out_bf16 else torch.float32)
+    lib = fv_sdpa.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    scale = 1.0 / d ** 0.5
+
+    def step():
+        if bt:
+            rc = lib.fv_sdpa_block_causal_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                               args.out_bf16, h, sq, sk, d, scale, bt, 0, 0, stream)
+        else:
+            rc = lib.fv_sdpa_dense_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                        args.out_bf16, h, sq, sk, d, scale, stream)
+        if rc != 0:
+            raise RuntimeError(f"kernel rc={rc}: {lib.fv_sdpa_last_error().decode()}")
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # whole-region wall clock, bracketed by synchronisation on both sides
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in evs:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kern_ms = sorted(a.elapsed_time(b) for a, b in evs)
+    avg_kernel_ms = sum(kern_ms) / len(kern_ms)
+    ms_per_step = wall * 1e3 / args.steps
+
+    flops = 4.0 * h * visible_pairs(sq, sk, bt) * d
+    flops_dense_equiv = 4.0 * h * sq * sk * d
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
+    bytes_min = 2.0 * (2 * h * sq * d + 2 * h * sk * d)
+
+    rec = {
+        "metric": "SDPA TFLOP/s + % bf16 MFMA peak, Wan-1.3B 480p self-attn (S=32760,H=12,d=128)"
+        if args.workload == "self" else f"SDPA TFLOP/s ({args.workload})",
+        "value": round(value, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": desc, "H": h, "Sq": sq, "Sk": sk, "d": d, "block_tokens": bt,
+                   "out": "bf16" if args.out_bf16 else "f32", "flops_per_call": flops,
+                   "dense_equivalent_flops": flops_dense_equiv},
+        "pct_of_bf16_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "flash_fwd_d128<causal>" if bt else "flash_fwd_d128",
+                     "avg_kernel_ms": round(avg_kernel_ms, 4), "median_kernel_ms": round(kern_ms[len(kern_ms) // 2], 4),
+                     "min_hbm_bytes": bytes_min,
+                     "hbm_frac_at_min_traffic": round(bytes_min / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+    }
+    if args.cpu_seconds > 0:
+        rec["cpu_baseline"] = cpu_baseline(h, sq, sk, d, bt, flops, q, k, v, args.cpu_seconds)
+    print(json.dumps(rec), flush=True)
+
+
+if __name__ == "__main__":
+    main()
