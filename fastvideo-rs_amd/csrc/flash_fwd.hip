@@ -80,7 +80,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const FlashParams p) {
         sink_tok = (int)min((long)sk, (long)p.sink * ft);
         const int sink_tiles = (sink_tok + kBN - 1) / kBN;
         mlo = lo_tok / kBN;
-        const int mhi = (hi_tok + kBN - 1) / kBN;
+        // sink blocks are visible to every query, also to those before them
+        const int mhi = max((hi_tok + kBN - 1) / kBN, sink_tiles);
         ns = min(sink_tiles, mlo);
         ne = ns + (mhi - mlo);
         const int tq = (q0 + wave * 32 + c32) / ft;

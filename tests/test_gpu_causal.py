@@ -1,0 +1,111 @@
+"""Parity of the block-causal flash kernel against the oracle (masked composed
+fp32 SDPA and the f64 checker). Cases follow the reference's wan_causal_attn
+table (crates/fastvideo-gpucheck/src/kernels_wan.rs:90-169; its d = 64 rows are
+run at d = 128 here), limit max|delta| <= 1e-2 and cosine >= 0.9999 (the
+reference's own limit is 2e-2), plus the schedule invariant of
+kernels_wan.rs:230-261: one block spanning the sequence is bit-identical to the
+dense kernel.
+"""
+import numpy as np
+import pytest
+
+from util import announce, assert_parity, qkv, sample_rows, to_dev_bf16
+
+pytestmark = pytest.mark.gpu
+
+CASES = [  # (bh, s, block_tokens, window, sink)
+    (2, 300, 60, 0, 0),
+    (6, 257, 37, 2, 0),
+    (2, 511, 50, 3, 1),
+    (4, 190, 19, 0, 2),
+    (1, 129, 1, 0, 0),
+    (2, 640, 128, 1, 0),
+    (2, 96, 200, 0, 0),
+    (2, 1000, 64, 2, 3),
+    (1, 777, 100, 1, 0),
+]
+
+
+@pytest.fixture(scope="module")
+def fv():
+    import torch
+
+    assert torch.cuda.is_available()
+    import fv_sdpa
+
+    fv_sdpa.lib()
+    return fv_sdpa
+
+
+@pytest.mark.parametrize("bh,s,bt,win,sink", CASES)
+def test_block_causal_matches_masked_oracle(fv, oracle, bh, s, bt, win, sink):
+    import torch
+
+    d, seed = 128, 3000 + s
+    announce(f"causal bh={bh} s={s} block={bt} window={win} sink={sink} seed={seed}")
+    q, k, v = qkv(seed, bh, s, s, d)
+    mask = oracle.block_causal_dense_mask(bt, win, sink, s, s)
+    want = oracle.sdpa_composed(q, k, v, mask=mask)
+    want64 = oracle.sdpa_f64(q, k, v, mask_bc=(bt, win, sink))
+    qd, kd, vd = (to_dev_bf16(x) for x in (q, k, v))
+    got = fv.sdpa_block_causal_bf16(qd, kd, vd, bt, win, sink)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    assert_parity(got, want, f"causal_{s}_{bt}_{win}_{sink}_vs_composed")
+    assert_parity(got, want64, f"causal_{s}_{bt}_{win}_{sink}_vs_f64")
+    got16 = fv.sdpa_block_causal_bf16(qd, kd, vd, bt, win, sink, out_bf16=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(got16.float().cpu().numpy(), oracle.quantize_bf16(got))
+
+
+def test_one_block_spanning_the_sequence_is_the_dense_kernel(fv):
+    import torch
+
+    bh, s, d = 3, 700, 128
+    announce("causal one-block == dense, 3x700")
+    q, k, v = (to_dev_bf16(x) for x in qkv(11, bh, s, s, d))
+    dense = fv.sdpa_dense_bf16(q, k, v)
+    causal = fv.sdpa_block_causal_bf16(q, k, v, 4096, 0, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(dense, causal)
+
+
+def test_sq_ne_sk_and_first_block_rows(fv, oracle):
+    import torch
+
+    # queries of a later chunk against a longer key sequence is not a reference
+    # case (its causal calls are square); square only, but check block-0 rows
+    # see only block 0 (kernel never loads later tiles for them)
+    bh, s, d, bt = 1, 512, 128, 128
+    announce("causal first-block rows 1x512")
+    q, k, v = qkv(13, bh, s, s, d)
+    got = fv.sdpa_block_causal_bf16(*(to_dev_bf16(x) for x in (q, k, v)), bt, 0, 0)
+    torch.cuda.synchronize()
+    want0 = oracle.sdpa_composed(q[:, :bt], k[:, :bt], v[:, :bt])
+    assert_parity(got[:, :bt].cpu().numpy(), want0, "causal_block0_rows")
+
+
+def test_declines(fv):
+    import torch
+
+    y = torch.zeros((1, 4, 128), device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(fv.FvDeclined):
+        fv.sdpa_block_causal_bf16(y, y, y, 0, 0, 0)
+
+
+@pytest.mark.parametrize("bt", [1560, 4680])
+def test_headline_causal_shape_sampled_rows(fv, oracle, bt):
+    """BASELINE config 3 at full size (21 frames x 1560 tokens) and the
+    reference's own 3-frame blocks; parity on sampled rows incl. frame edges."""
+    import torch
+
+    bh, s, d = 12, 32760, 128
+    announce(f"causal headline bh={bh} s={s} block={bt}")
+    g = torch.Generator(device="cuda").manual_seed(77)
+    q, k, v = (torch.randn((bh, s, d), generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    out = fv.sdpa_block_causal_bf16(q, k, v, bt, 0, 0)
+    torch.cuda.synchronize()
+    rows = sample_rows(3, s, 24, extra=(0, bt - 1, bt, 2 * bt - 1, 2 * bt, 10 * bt + 5, s - bt, s - 1))
+    want = oracle.sdpa_composed_rows(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), rows,
+                                     mask_bc=(bt, 0, 0))
+    assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, f"causal_headline_{bt}")
