@@ -1,0 +1,194 @@
+// Building blocks shared by the gfx950 attention kernels that stage K/V tiles
+// with direct global->LDS loads (global_load_lds_dwordx4) into XOR-swizzled,
+// unpadded [64 keys][128 d] bf16 tiles.
+//
+// LDS tile layout (16 KB): row r is 256 B = 16 chunks of 16 B; logical chunk c
+// of row r lives at chunk position c ^ swz(r), with
+//   K tiles: swz(r) = r & 15        (32 consecutive keys reading one chunk
+//                                    column hit 16 distinct positions)
+//   V tiles: swz(r) = (r & 3) << 2  (the 4 rows of a transposed 4x16 read land
+//                                    in 4 disjoint 64 B bank groups)
+// The LDS-DMA write puts lane i's 16 B at base + 16 i, so the swizzle is applied
+// on the global side: lane i fetches the chunk that belongs at its position.
+#pragma once
+#include "fv_common.h"
+
+namespace fv {
+
+constexpr int kTileRows = 64;
+constexpr int kRowBytes = 256;
+constexpr int kTileBytes = kTileRows * kRowBytes;   // 16 KB
+
+typedef __attribute__((address_space(1))) void glb_void;
+typedef __attribute__((address_space(3))) void lds_void;
+
+// One wave-wide LDS-DMA instruction: lane i copies 16 B from its own global
+// address to LDS byte address lds_base + 16 i (lds_base wave-uniform). Issued as
+// inline asm so that the compiler's wait-count insertion does not serialise
+// later LDS reads of OTHER buffers behind it; the kernels order these loads with
+// wait_vmcnt<N>() + block_barrier() themselves.
+FV_DEV void lds_dma16(unsigned lds_base, const void* gptr) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, off"
+        :
+        : "s"(lds_base), "v"(gptr)
+        : "memory", "m0");
+}
+
+// Workgroup barrier without the memory fences of __syncthreads() (a fence
+// would wait for every outstanding LDS-DMA load, defeating the prefetch). LDS
+// reads issued before it have been consumed by then (their MFMA waited on them).
+FV_DEV void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// s_waitcnt vmcnt(N) alone (expcnt / lgkmcnt untouched), gfx9 encoding.
+template <int N>
+FV_DEV void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is 6 bits");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Issue the asynchronous loads of one 64 x 128 bf16 tile whose rows are
+// contiguous in global memory (256 B apart). NW waves share the tile, 4 rows
+// per wave instruction. Rows >= rows_valid re-read the last valid row (the
+// caller masks their scores to -inf, so their content only has to be finite
+// data the tensor already holds). Completion is tracked by vmcnt: 16 / NW
+// instructions per wave and tile.
+template <int NW, bool IS_V>
+FV_DEV void tile_load_async(lds_u8* buf, const uint16_t* g, int rows_valid, int wave, int lane) {
+    constexpr int ITER = 16 / NW;
+    const int p = lane & 15;
+    const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 4 * kRowBytes);
+#pragma unroll
+    for (int it = 0; it < ITER; it++) {
+        const int R = (wave * ITER + it) * 4;
+        const int r = R + (lane >> 4);
+        const int c = IS_V ? (p ^ ((r & 3) << 2)) : (p ^ (r & 15));
+        const int rs = min(r, rows_valid - 1);
+        lds_dma16(base + it * 4 * kRowBytes, g + (size_t)rs * 128 + c * 8);
+    }
+}
+
+// Per-lane read bases into a swizzled tile.
+struct TileReadBases {
+    int k;   // K A-operand: ^ (dk << 5), + kb * 32 rows
+    int v;   // V^T A-operand (transposed read): ^ (db << 6), + (16 t + 8 g) rows
+};
+FV_DEV TileReadBases tile_read_bases(int lane) {
+    const int h = lane >> 5, c32 = lane & 31;
+    const int b16 = lane >> 4, i16 = lane & 15;
+    TileReadBases b;
+    b.k = c32 * kRowBytes + ((((c32 & 15) ^ h)) << 4);
+    const int r = 4 * h + (i16 >> 2);
+    const int c_lane = 2 * (b16 & 1) + ((i16 & 3) >> 1);
+    b.v = r * kRowBytes + ((((i16 >> 2) << 2) + c_lane) << 4) + 8 * (i16 & 1);
+    return b;
+}
+
+// S^T (64 keys x 32 queries) = K Q^T for one wave: s[b][i] is key
+// 32 b + 8 (i/4) + 4 (lane/32) + i%4 of the tile, query lane%32.
+FV_DEV void qk_tile(const lds_u8* kb, int k_base, const bf16x8 (&qf)[8], f32x16 (&s)[2]) {
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[b][i] = 0.f;
+#pragma unroll
+        for (int dk = 0; dk < 8; dk++) {
+            const bf16x8 a = lds_read_b128(kb + (k_base ^ (dk << 5)) + b * 32 * kRowBytes);
+            s[b] = mfma32(a, qf[dk], s[b]);
+        }
+    }
+}
+
+// Online-softmax state of one query (replicated in lanes l and l^32; l_acc is
+// the lane's own share of the row sum).
+struct SoftmaxState {
+    float m_run, m_used, ms_used, l_acc;
+    FV_DEV void init() {
+        m_run = neg_inf();
+        m_used = neg_inf();
+        ms_used = 0.f;
+        l_acc = 0.f;
+    }
+};
+
+constexpr float kRescaleLog2 = 6.0f;
+
+// Row max, lazy rescale of (l, O), P = 2^(s*sl2 - offset), bf16 pack.
+// pb[t] is the B operand (16 key slots x 32 queries) for key group t.
+FV_DEV void softmax_tile(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float sl2,
+                         bf16x8 (&pb)[4]) {
+    const float NEG = neg_inf();
+    float mx = s[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s[0][i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s[1][i]);
+    mx = pair_max(mx);
+    st.m_run = __builtin_fmaxf(st.m_run, mx);
+    const bool need = (st.m_run * sl2 - st.ms_used > kRescaleLog2) ||
+                      (st.m_used == NEG && st.m_run != NEG);
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {
+        const float ms_new = (st.m_run == NEG) ? 0.f : st.m_run * sl2;
+        const float alpha = (st.m_used == NEG) ? 0.f : fast_exp2(st.ms_used - ms_new);
+        st.l_acc *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
+        st.m_used = st.m_run;
+        st.ms_used = ms_new;
+    }
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+        f32x16 e;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            e[i] = fast_exp2(__builtin_fmaf(s[b][i], sl2, -st.ms_used));
+            st.l_acc += e[i];
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            f32x8 f;
+#pragma unroll
+            for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
+            pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
+        }
+    }
+}
+
+// O^T (128 d x 32 queries) += V^T P^T.
+FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 (&o)[4]) {
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+#pragma unroll
+        for (int db = 0; db < 4; db++) {
+            const int a0 = (v_base ^ (db << 6)) + (16 * t) * kRowBytes;
+            const s16x4 lo = lds_read_tr16_b64(vb + a0);
+            const s16x4 hi = lds_read_tr16_b64(vb + a0 + 8 * kRowBytes);
+            s16x8 a;
+            a.lo = lo;
+            a.hi = hi;
+            o[db] = mfma32(__builtin_bit_cast(bf16x8, a), pb[t], o[db]);
+        }
+    }
+}
+
+// Q^T fragments for the wave's 32 queries: rows row0 + lane%32 of a row-major
+// [rows][128] bf16 tensor; rows >= nrows read as zero.
+FV_DEV void load_q_frags(const uint16_t* q, int row, bool ok, int lane, bf16x8 (&qf)[8]) {
+    const uint16_t* src = q + (size_t)row * 128 + 8 * (lane >> 5);
+#pragma unroll
+    for (int dk = 0; dk < 8; dk++) {
+        u32x4 t = {0u, 0u, 0u, 0u};
+        if (ok) t = *reinterpret_cast<const u32x4*>(src + 16 * dk);
+        qf[dk] = __builtin_bit_cast(bf16x8, t);
+    }
+    // Drain these (compiler-tracked) loads here: a wait the compiler would
+    // otherwise place inside the main loop also counts the untracked LDS-DMA
+    // loads in flight there and would stall on them.
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+}
+
+}  // namespace fv

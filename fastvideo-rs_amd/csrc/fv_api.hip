@@ -10,21 +10,27 @@
 #include "fv_common.h"
 #include "fv_internal.h"
 
-namespace {
+static thread_local std::string g_last_error;
 
-thread_local std::string g_last_error;
-
-int fail_hip(hipError_t e, const char* what) {
+int fv_fail_hip(hipError_t e, const char* what) {
     char buf[256];
     snprintf(buf, sizeof buf, "%s: %s (hipError %d)", what, hipGetErrorString(e), (int)e);
     g_last_error = buf;
     return -(int)e;
 }
-
-int decline(const char* why) {
+int fv_decline(const char* why) {
     g_last_error = why;
     return FV_DECLINED;
 }
+int fv_invalid(const char* why) {
+    g_last_error = why;
+    return -(int)hipErrorInvalidValue;
+}
+
+namespace {
+
+int fail_hip(hipError_t e, const char* what) { return fv_fail_hip(e, what); }
+int decline(const char* why) { return fv_decline(why); }
 
 __global__ void cast_f32_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y,
                                      size_t n) {
@@ -51,10 +57,7 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
                  bool causal, size_t block_tokens, size_t window, size_t sink, void* stream) {
     if (!fv_sdpa_supported(1, bh, sq, sk, d)) return decline("sdpa: shape not taken by the fused kernel");
     if (!(scale > 0.0f) || !(scale < 3.0e38f)) return decline("sdpa: the fused kernel needs a finite scale > 0");
-    if (!q || !k || !v || !out) {
-        g_last_error = "sdpa: null operand";
-        return -(int)hipErrorInvalidValue;
-    }
+    if (!q || !k || !v || !out) return fv_invalid("sdpa: null operand");
     fv::FlashParams p;
     p.q = q;
     p.k = k;

@@ -21,7 +21,43 @@ struct FlashParams {
     int ft, win, sink;  // block-causal: block tokens, window blocks, sink blocks
 };
 
+struct VsaFineParams {
+    const uint16_t* qt;           // tile-ordered bf16 [bh, nb*64, 128]
+    const uint16_t* kt;
+    const uint16_t* vt;
+    const unsigned* selected;     // [bh, nb, topk]
+    const int* block_sizes;       // [nb]
+    float* out;                   // [bh, q_tiles*64, 128] f32, tile-slot order
+    int num_tiles, topk;
+    float sl2;
+    int q_base, q_tiles;          // query tiles [q_base, q_base + q_tiles)
+    int total, per_xcd;           // bh * q_tiles, ceil(total / 8)
+};
+
 }  // namespace fv
 
 extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal,
                                                hipStream_t stream);
+extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16, const int* slot_src,
+                                                   const int* block_sizes, float* out, size_t bh,
+                                                   size_t seq, int dim, int num_tiles, int round16,
+                                                   hipStream_t st);
+extern "C" hipError_t fv_internal_launch_coarse(const float* qc, const float* kc, const float* vc,
+                                                float* scores, float* coarse, size_t bh, int nb,
+                                                int dim, float scale, hipStream_t st);
+extern "C" hipError_t fv_internal_launch_topk(const float* scores, unsigned* out, int rows, int n, int k,
+                                              hipStream_t st);
+extern "C" hipError_t fv_internal_launch_tile_qkv(const void* x, int x_is_bf16, const int* slot_src,
+                                                  uint16_t* xt, size_t bh, size_t seq, size_t padded,
+                                                  int dim, hipStream_t st);
+extern "C" hipError_t fv_internal_launch_fine(const fv::VsaFineParams* p, hipStream_t st);
+extern "C" hipError_t fv_internal_launch_combine(const float* sparse, const float* coarse,
+                                                 const void* gate, int gate_is_bf16,
+                                                 const int* slot_src, float* out, size_t bh,
+                                                 size_t seq, int num_tiles, int q_base, int q_tiles,
+                                                 hipStream_t st);
+
+// Error plumbing of the C ABI (defined in fv_api.hip): the message is kept per thread.
+int fv_fail_hip(hipError_t e, const char* what);   // returns -(int)e
+int fv_decline(const char* why);                    // returns FV_DECLINED
+int fv_invalid(const char* why);                    // returns -(int)hipErrorInvalidValue

@@ -1,0 +1,521 @@
+// Video Sparse Attention stages for gfx950: tile mean, coarse scores, coarse
+// softmax x V, radix-select top-k, tile permute, block-sparse fine attention,
+// gated combine. Reference stages: crates/fastvideo-cudarc/src/rt/vsa.rs:358-470
+// and the kernels cited per function below (kernels/core.cu, kernels/attn3.cu).
+#include "attn_core.h"
+#include "fv_internal.h"
+
+namespace fv {
+
+constexpr int kTileElems = 64;   // VSA cube = 4x4x4 tokens (rt/vsa.rs:29-31)
+
+// ---- tile mean (kernels/core.cu:550-570, kernels/attn3.cu:208-226) --------------
+// One 32-lane group per tile, 4 consecutive d per lane; the sum runs over the
+// tile's real tokens in slot order with one f32 add per token, then / n — the
+// same order and operations as the reference, so the result is bit-identical
+// to its host restatement.
+template <bool IN_BF16>
+__global__ __launch_bounds__(256) void vsa_tile_mean_kernel(
+    const void* __restrict__ x, const int* __restrict__ slot_src,
+    const int* __restrict__ block_sizes, float* __restrict__ out, long seq, int dim,
+    int num_tiles, int round16) {
+    const int grp = threadIdx.x >> 5, ln = threadIdx.x & 31;
+    const int tile = blockIdx.x * 8 + grp;
+    const long bh = blockIdx.y;
+    if (tile >= num_tiles) return;
+    const int n = block_sizes[tile];
+    const int* src = slot_src + (long)tile * kTileElems;
+    float* ob = out + (bh * num_tiles + tile) * (long)dim;
+    for (int d0 = ln * 4; d0 < dim; d0 += 128) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < n; j++) {
+            const long tok = src[j];
+            f32x4 v;
+            if constexpr (IN_BF16) {
+                const u32x2 raw = *reinterpret_cast<const u32x2*>(
+                    (const uint16_t*)x + (bh * seq + tok) * dim + d0);
+                v[0] = __builtin_bit_cast(float, raw[0] << 16);
+                v[1] = __builtin_bit_cast(float, raw[0] & 0xffff0000u);
+                v[2] = __builtin_bit_cast(float, raw[1] << 16);
+                v[3] = __builtin_bit_cast(float, raw[1] & 0xffff0000u);
+            } else {
+                v = *reinterpret_cast<const f32x4*>((const float*)x + (bh * seq + tok) * dim + d0);
+                if (round16) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] = bf16_bits_to_f32(bf16_rne_bits(v[e]));
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[e] = __fadd_rn(acc[e], v[e]);
+        }
+        f32x4 r;
+#pragma unroll
+        for (int e = 0; e < 4; e++) r[e] = n > 0 ? __fdiv_rn(acc[e], (float)n) : 0.0f;
+        *reinterpret_cast<f32x4*>(ob + d0) = r;
+    }
+}
+
+// ---- coarse scores (rt/vsa.rs:385-388) ---------------------------------------------
+// scores[bh, qt, kt] = (sum over d ascending of qc*kc, f32 mul then add) * scale.
+// The reference runs cuBLAS f32 here; a fixed summation order makes the scores,
+// and so the top-k selection, reproducible bit for bit on the host.
+__global__ __launch_bounds__(256) void vsa_coarse_scores_kernel(
+    const float* __restrict__ qc, const float* __restrict__ kc, float* __restrict__ scores,
+    int nb, int dim, float scale) {
+#pragma clang fp contract(off)   // keep mul and add separate: the order is part of the contract
+    __shared__ float qs[64][33];
+    __shared__ float ks[64][33];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int q0 = blockIdx.y * 64, k0 = blockIdx.x * 64;
+    const long bh = blockIdx.z;
+    const float* qb = qc + bh * nb * (long)dim;
+    const float* kb = kc + bh * nb * (long)dim;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = 0.f;
+    for (int d0 = 0; d0 < dim; d0 += 32) {
+        for (int e = threadIdx.x; e < 64 * 32; e += 256) {
+            const int r = e >> 5, c = e & 31;
+            qs[r][c] = (q0 + r < nb && d0 + c < dim) ? qb[(long)(q0 + r) * dim + d0 + c] : 0.f;
+            ks[r][c] = (k0 + r < nb && d0 + c < dim) ? kb[(long)(k0 + r) * dim + d0 + c] : 0.f;
+        }
+        __syncthreads();
+        const int dn = min(32, dim - d0);
+        for (int c = 0; c < dn; c++) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) a[i] = qs[ty * 4 + i][c];
+#pragma unroll
+            for (int j = 0; j < 4; j++) b[j] = ks[tx * 4 + j][c];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = acc[i][j] + a[i] * b[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int qi = q0 + ty * 4 + i, kj = k0 + tx * 4 + j;
+            if (qi < nb && kj < nb) scores[(bh * nb + qi) * (long)nb + kj] = acc[i][j] * scale;
+        }
+}
+
+// ---- coarse softmax x V (rt/vsa.rs:389-393, kernels/core.cu:177-252) ---------------
+// coarse[bh, qt, :] = softmax(scores[bh, qt, :]) vc[bh]; four query tiles per block
+// share every vc row they read. dim = 128.
+constexpr int kCoarseRows = 4;
+__global__ __launch_bounds__(256) void vsa_coarse_pv_kernel(
+    const float* __restrict__ scores, const float* __restrict__ vc, float* __restrict__ coarse,
+    int nb) {
+    extern __shared__ float p_lds[];   // [kCoarseRows][nb]
+    __shared__ float red[kCoarseRows][4];
+    __shared__ float stat[kCoarseRows];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q0 = blockIdx.x * kCoarseRows;
+    const long bh = blockIdx.y;
+    const int rows = min(kCoarseRows, nb - q0);
+    const float* sb = scores + (bh * nb + q0) * (long)nb;
+    for (int e = tid; e < rows * nb; e += 256) p_lds[e] = sb[e];
+    __syncthreads();
+    // row max
+    for (int r = 0; r < rows; r++) {
+        float m = neg_inf();
+        for (int j = tid; j < nb; j += 256) m = fmaxf(m, p_lds[r * nb + j]);
+        for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+        if (lane == 0) red[r][wave] = m;
+    }
+    __syncthreads();
+    if (tid < rows) stat[tid] = fmaxf(fmaxf(red[tid][0], red[tid][1]), fmaxf(red[tid][2], red[tid][3]));
+    __syncthreads();
+    for (int r = 0; r < rows; r++) {
+        const float m = stat[r];
+        float s = 0.f;
+        for (int j = tid; j < nb; j += 256) {
+            const float e = expf(p_lds[r * nb + j] - m);
+            p_lds[r * nb + j] = e;
+            s += e;
+        }
+        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+        if (lane == 0) red[r][wave] = s;
+    }
+    __syncthreads();
+    if (tid < rows) stat[tid] = 1.0f / (red[tid][0] + red[tid][1] + red[tid][2] + red[tid][3]);
+    __syncthreads();
+    // each half-block owns two rows; lane d accumulates over all key tiles
+    const int d = tid & 127, rh = tid >> 7;
+    const float* vb = vc + bh * nb * 128L + d;
+    float a0 = 0.f, a1 = 0.f;
+    const float* p0 = p_lds + (2 * rh) * nb;
+    const float* p1 = p_lds + (2 * rh + 1) * nb;
+    const bool ok0 = 2 * rh < rows, ok1 = 2 * rh + 1 < rows;
+    if (ok0) {
+        for (int kt = 0; kt < nb; kt++) {
+            const float vv = vb[(long)kt * 128];
+            a0 += p0[kt] * vv;
+            if (ok1) a1 += p1[kt] * vv;
+        }
+        coarse[(bh * nb + q0 + 2 * rh) * 128L + d] = a0 * stat[2 * rh];
+        if (ok1) coarse[(bh * nb + q0 + 2 * rh + 1) * 128L + d] = a1 * stat[2 * rh + 1];
+    }
+}
+
+// ---- top-k (kernels/core.cu:576-619, kernels/attn3.cu:279-363) ----------------------
+// T = k-th largest sortable key of the row (8-bit radix select, 4 histogram
+// passes over the row held in LDS); output = indices with key > T ascending,
+// then key == T ascending, up to k, zero padded. Bit-exact integer work.
+FV_DEV unsigned sortable_key(float x) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+constexpr int kTopkMaxN = 4096;
+
+__global__ __launch_bounds__(256) void vsa_topk_kernel(const float* __restrict__ scores,
+                                                       unsigned* __restrict__ out, int rows,
+                                                       int n, int k) {
+    __shared__ unsigned keys[kTopkMaxN];
+    __shared__ unsigned hist[256];
+    __shared__ unsigned sel_prefix, sel_rem;
+    __shared__ unsigned wsum_gt[4], wsum_eq[4];
+    const int row = blockIdx.x;
+    if (row >= rows) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float* s = scores + (long)row * n;
+    for (int i = tid; i < n; i += 256) keys[i] = sortable_key(s[i]);
+    if (tid == 0) {
+        sel_prefix = 0u;
+        sel_rem = (unsigned)k;
+    }
+    __syncthreads();
+    unsigned thr = 0u;
+    if (k <= n) {
+#pragma unroll 1
+        for (int pass = 0; pass < 4; pass++) {
+            const int shift = 24 - 8 * pass;
+            const unsigned hi_mask = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8));
+            hist[tid] = 0u;
+            __syncthreads();
+            const unsigned prefix = sel_prefix;
+            for (int i = tid; i < n; i += 256) {
+                const unsigned key = keys[i];
+                if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+            }
+            __syncthreads();
+            if (wave == 0) {
+                // lane l owns bins [4l, 4l+4); suffix counts from the top bin down
+                unsigned c[4];
+#pragma unroll
+                for (int b = 0; b < 4; b++) c[b] = hist[lane * 4 + b];
+                const unsigned local = c[0] + c[1] + c[2] + c[3];
+                unsigned suffix = local;
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const unsigned o = __shfl_down(suffix, off);
+                    if (lane + off < 64) suffix += o;
+                }
+                const unsigned rem = sel_rem;
+                const unsigned above = suffix - local;
+                if (above < rem && suffix >= rem) {
+                    unsigned acc = above;
+                    int b = 3;
+                    for (; b > 0; b--) {
+                        if (acc + c[b] >= rem) break;
+                        acc += c[b];
+                    }
+                    sel_prefix = prefix | ((unsigned)(lane * 4 + b) << shift);
+                    sel_rem = rem - acc;
+                }
+            }
+            __syncthreads();
+        }
+        thr = sel_prefix;
+    }
+    // ordered compaction: thread t owns the contiguous index range [t*C, (t+1)*C)
+    const int C = (n + 255) / 256;
+    const int i0 = min(n, tid * C), i1 = min(n, i0 + C);
+    unsigned cgt = 0, ceq = 0;
+    for (int i = i0; i < i1; i++) {
+        const unsigned key = keys[i];
+        cgt += key > thr;
+        ceq += key == thr;
+    }
+    // exclusive scans over the block
+    unsigned sgt = cgt, seq_ = ceq;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned a = __shfl_up(sgt, off), b = __shfl_up(seq_, off);
+        if (lane >= off) {
+            sgt += a;
+            seq_ += b;
+        }
+    }
+    if (lane == 63) {
+        wsum_gt[wave] = sgt;
+        wsum_eq[wave] = seq_;
+    }
+    __syncthreads();
+    unsigned base_gt = 0, base_eq = 0, tot_gt = 0, tot_eq = 0;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        if (w < wave) {
+            base_gt += wsum_gt[w];
+            base_eq += wsum_eq[w];
+        }
+        tot_gt += wsum_gt[w];
+        tot_eq += wsum_eq[w];
+    }
+    unsigned pgt = base_gt + sgt - cgt;
+    unsigned peq = tot_gt + base_eq + seq_ - ceq;
+    unsigned* dst = out + (long)row * k;
+    for (int i = i0; i < i1; i++) {
+        const unsigned key = keys[i];
+        if (key > thr) {
+            if (pgt < (unsigned)k) dst[pgt] = (unsigned)i;
+            pgt++;
+        } else if (key == thr) {
+            if (peq < (unsigned)k) dst[peq] = (unsigned)i;
+            peq++;
+        }
+    }
+    for (unsigned pos = tot_gt + tot_eq + tid; pos < (unsigned)k; pos += 256) dst[pos] = 0u;
+}
+
+// ---- tile permute (kernels/core.cu:1659-1672, kernels/attn3.cu:230-244) --------------
+// [bh, seq, 128] -> tile-contiguous bf16 [bh, padded, 128]; padding slots are zero.
+template <bool IN_BF16>
+__global__ __launch_bounds__(256) void vsa_tile_qkv_kernel(const void* __restrict__ x,
+                                                           const int* __restrict__ slot_src,
+                                                           uint16_t* __restrict__ xt, long seq,
+                                                           long padded, int dim) {
+    const long chunks = dim / 8;
+    const long rem = blockIdx.x * 256L + threadIdx.x;
+    if (rem >= padded * chunks) return;
+    const long bh = blockIdx.y;
+    const long slot = rem / chunks;
+    const long c = rem - slot * chunks;
+    const int src = slot_src[slot];
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (src >= 0) {
+        if constexpr (IN_BF16) {
+            v = *reinterpret_cast<const u32x4*>((const uint16_t*)x + (bh * seq + src) * dim + c * 8);
+        } else {
+            const float* px = (const float*)x + (bh * seq + src) * dim + c * 8;
+            const f32x4 a = *reinterpret_cast<const f32x4*>(px);
+            const f32x4 b = *reinterpret_cast<const f32x4*>(px + 4);
+            v[0] = bf16_rne_bits(a[0]) | ((unsigned)bf16_rne_bits(a[1]) << 16);
+            v[1] = bf16_rne_bits(a[2]) | ((unsigned)bf16_rne_bits(a[3]) << 16);
+            v[2] = bf16_rne_bits(b[0]) | ((unsigned)bf16_rne_bits(b[1]) << 16);
+            v[3] = bf16_rne_bits(b[2]) | ((unsigned)bf16_rne_bits(b[3]) << 16);
+        }
+    }
+    *reinterpret_cast<u32x4*>(xt + (bh * padded + slot) * dim + c * 8) = v;
+}
+
+// ---- fine stage (kernels/core.cu:1029-1179) ---------------------------------------------
+// One workgroup (2 waves x 32 queries) per (query tile, batch*head): online
+// softmax over the selected key tiles in list order; key columns >=
+// block_sizes[tile] are -inf. K and V tiles are separate single LDS buffers fed
+// by direct global->LDS loads: K(i+1) streams in under softmax/PV of tile i and
+// V(i) under QK/softmax of tile i. 32 KB of LDS per workgroup, so four
+// workgroups share a CU.
+__global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    lds_u8* kbuf = (lds_u8*)smem_raw;
+    lds_u8* vbuf = kbuf + kTileBytes;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int h = lane >> 5, c32 = lane & 31;
+    const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (work >= p.total) return;
+    const int bh = work / p.q_tiles;
+    const int qtile = p.q_base + work % p.q_tiles;
+    if (qtile >= p.num_tiles) return;
+    const int nb = p.num_tiles, topk = p.topk;
+    const size_t padded = (size_t)nb * kTileElems;
+    const uint16_t* kb = p.kt + (size_t)bh * padded * 128;
+    const uint16_t* vb = p.vt + (size_t)bh * padded * 128;
+    const unsigned* sel = p.selected + ((size_t)bh * nb + qtile) * topk;
+    const float sl2 = p.sl2;
+    const float NEG = neg_inf();
+
+    bf16x8 qf[8];
+    load_q_frags(p.qt + ((size_t)bh * padded + (size_t)qtile * kTileElems) * 128, wave * 32 + c32,
+                 true, lane, qf);
+    const TileReadBases rb = tile_read_bases(lane);
+
+    f32x16 o[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[db][i] = 0.f;
+    SoftmaxState st;
+    st.init();
+
+    int tile = min((int)sel[0], nb - 1);
+    tile_load_async<2, false>(kbuf, kb + (size_t)tile * kTileElems * 128, kTileElems, wave, lane);
+#pragma unroll 1
+    for (int i = 0; i < topk; i++) {
+        const int valid = p.block_sizes[tile];
+        wait_vmcnt<0>();     // K(i) landed
+        block_barrier();     // ... for every wave; PV(i-1) finished everywhere: V buffer free
+        tile_load_async<2, true>(vbuf, vb + (size_t)tile * kTileElems * 128, kTileElems, wave, lane);
+        f32x16 s[2];
+        qk_tile(kbuf, rb.k, qf, s);
+        block_barrier();     // K buffer free
+        const bool more = i + 1 < topk;
+        if (more) {
+            tile = min((int)sel[i + 1], nb - 1);
+            tile_load_async<2, false>(kbuf, kb + (size_t)tile * kTileElems * 128, kTileElems, wave, lane);
+        }
+        if (valid < kTileElems) {
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int col = 32 * b + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (col >= valid) s[b][e] = NEG;
+                }
+        }
+        bf16x8 pb[4];
+        softmax_tile(s, st, o, sl2, pb);
+        if (more) wait_vmcnt<8>(); else wait_vmcnt<0>();   // V(i) landed; K(i+1) may be in flight
+        block_barrier();
+        pv_tile(vbuf, rb.v, pb, o);
+    }
+
+    const float l_tot = pair_sum(st.l_acc);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    float* ob = p.out + (((size_t)bh * p.q_tiles + (qtile - p.q_base)) * kTileElems + wave * 32 + c32) * 128;
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            f32x4 r;
+#pragma unroll
+            for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
+            *reinterpret_cast<f32x4*>(ob + 32 * db + 8 * g + 4 * h) = r;
+        }
+}
+
+// ---- combine (kernels/core.cu:803-835) -----------------------------------------------------
+// out[token] = coarse[tile] * gate[token] + sparse[slot]; gate == null is a gate of one.
+template <bool GATE_BF16>
+__global__ __launch_bounds__(256) void vsa_combine_kernel(
+    const float* __restrict__ sparse, const float* __restrict__ coarse,
+    const void* __restrict__ gate, const int* __restrict__ slot_src, float* __restrict__ out,
+    long seq, int num_tiles, int q_base, int q_tiles, int has_gate) {
+#pragma clang fp contract(off)   // coarse * gate rounds to f32 before the add, as on the host
+    // one thread per (slot, 4 d): 32 threads per slot, 8 slots per block
+    const long slot_lin = blockIdx.x * 8L + (threadIdx.x >> 5);   // over q_tiles * 64
+    const int d0 = (threadIdx.x & 31) * 4;
+    const long bh = blockIdx.y;
+    if (slot_lin >= (long)q_tiles * kTileElems) return;
+    const int g = (int)(slot_lin / kTileElems);
+    const int tile = q_base + g;
+    if (tile >= num_tiles) return;
+    const int src = slot_src[(long)tile * kTileElems + (slot_lin - (long)g * kTileElems)];
+    if (src < 0) return;
+    const f32x4 sp = *reinterpret_cast<const f32x4*>(sparse + (bh * q_tiles * kTileElems + slot_lin) * 128 + d0);
+    const f32x4 co = *reinterpret_cast<const f32x4*>(coarse + (bh * num_tiles + tile) * 128L + d0);
+    f32x4 ga = {1.f, 1.f, 1.f, 1.f};
+    if (has_gate) {
+        if constexpr (GATE_BF16) {
+            const u32x2 raw = *reinterpret_cast<const u32x2*>((const uint16_t*)gate + (bh * seq + src) * 128 + d0);
+            ga[0] = __builtin_bit_cast(float, raw[0] << 16);
+            ga[1] = __builtin_bit_cast(float, raw[0] & 0xffff0000u);
+            ga[2] = __builtin_bit_cast(float, raw[1] << 16);
+            ga[3] = __builtin_bit_cast(float, raw[1] & 0xffff0000u);
+        } else {
+            ga = *reinterpret_cast<const f32x4*>((const float*)gate + (bh * seq + src) * 128 + d0);
+        }
+    }
+    f32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; e++) r[e] = co[e] * ga[e] + sp[e];
+    *reinterpret_cast<f32x4*>(out + (bh * seq + src) * 128 + d0) = r;
+}
+
+}  // namespace fv
+
+// ---- host launchers -----------------------------------------------------------------------
+
+using namespace fv;
+
+extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16, const int* slot_src,
+                                                   const int* block_sizes, float* out, size_t bh,
+                                                   size_t seq, int dim, int num_tiles, int round16,
+                                                   hipStream_t st) {
+    const dim3 grid((num_tiles + 7) / 8, (unsigned)bh), block(256);
+    if (x_is_bf16)
+        hipLaunchKernelGGL(vsa_tile_mean_kernel<true>, grid, block, 0, st, x, slot_src, block_sizes, out,
+                           (long)seq, dim, num_tiles, round16);
+    else
+        hipLaunchKernelGGL(vsa_tile_mean_kernel<false>, grid, block, 0, st, x, slot_src, block_sizes, out,
+                           (long)seq, dim, num_tiles, round16);
+    return hipGetLastError();
+}
+
+extern "C" hipError_t fv_internal_launch_coarse(const float* qc, const float* kc, const float* vc,
+                                                float* scores, float* coarse, size_t bh, int nb,
+                                                int dim, float scale, hipStream_t st) {
+    const dim3 g1((nb + 63) / 64, (nb + 63) / 64, (unsigned)bh);
+    hipLaunchKernelGGL(vsa_coarse_scores_kernel, g1, dim3(256), 0, st, qc, kc, scores, nb, dim, scale);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || !coarse) return e;
+    const size_t lds = sizeof(float) * kCoarseRows * (size_t)nb;
+    static bool attr_done = false;
+    if (!attr_done) {
+        e = hipFuncSetAttribute((const void*)vsa_coarse_pv_kernel,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, sizeof(float) * kCoarseRows * kTopkMaxN);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    const dim3 g2((nb + kCoarseRows - 1) / kCoarseRows, (unsigned)bh);
+    hipLaunchKernelGGL(vsa_coarse_pv_kernel, g2, dim3(256), lds, st, scores, vc, coarse, nb);
+    return hipGetLastError();
+}
+
+extern "C" hipError_t fv_internal_launch_topk(const float* scores, unsigned* out, int rows, int n, int k,
+                                              hipStream_t st) {
+    hipLaunchKernelGGL(vsa_topk_kernel, dim3(rows), dim3(256), 0, st, scores, out, rows, n, k);
+    return hipGetLastError();
+}
+
+extern "C" hipError_t fv_internal_launch_tile_qkv(const void* x, int x_is_bf16, const int* slot_src,
+                                                  uint16_t* xt, size_t bh, size_t seq, size_t padded,
+                                                  int dim, hipStream_t st) {
+    const size_t per = padded * (size_t)(dim / 8);
+    const dim3 grid((unsigned)((per + 255) / 256), (unsigned)bh), block(256);
+    if (x_is_bf16)
+        hipLaunchKernelGGL(vsa_tile_qkv_kernel<true>, grid, block, 0, st, x, slot_src, xt, (long)seq,
+                           (long)padded, dim);
+    else
+        hipLaunchKernelGGL(vsa_tile_qkv_kernel<false>, grid, block, 0, st, x, slot_src, xt, (long)seq,
+                           (long)padded, dim);
+    return hipGetLastError();
+}
+
+extern "C" hipError_t fv_internal_launch_fine(const fv::VsaFineParams* p, hipStream_t st) {
+    hipLaunchKernelGGL(vsa_fine_kernel, dim3(p->per_xcd * 8), dim3(128), 2 * kTileBytes, st, *p);
+    return hipGetLastError();
+}
+
+extern "C" hipError_t fv_internal_launch_combine(const float* sparse, const float* coarse,
+                                                 const void* gate, int gate_is_bf16,
+                                                 const int* slot_src, float* out, size_t bh,
+                                                 size_t seq, int num_tiles, int q_base, int q_tiles,
+                                                 hipStream_t st) {
+    const dim3 grid((unsigned)(((size_t)q_tiles * kTileElems + 7) / 8), (unsigned)bh), block(256);
+    const int has_gate = gate != nullptr;
+    if (gate_is_bf16)
+        hipLaunchKernelGGL(vsa_combine_kernel<true>, grid, block, 0, st, sparse, coarse, gate, slot_src, out,
+                           (long)seq, num_tiles, q_base, q_tiles, has_gate);
+    else
+        hipLaunchKernelGGL(vsa_combine_kernel<false>, grid, block, 0, st, sparse, coarse, gate, slot_src, out,
+                           (long)seq, num_tiles, q_base, q_tiles, has_gate);
+    return hipGetLastError();
+}

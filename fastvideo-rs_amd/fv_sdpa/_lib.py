@@ -26,6 +26,21 @@ SIGNATURES = {
                                             _sz, _sz, _sz, _vp]),
     "fv_cast_f32_bf16": (C.c_int, [_vp, _vp, _sz, _vp]),
     "fv_cast_bf16_f32": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "fv_vsa_topk_for": (_sz, [C.c_double, _sz]),
+    "fv_vsa_tile_plan": (C.c_int, [_sz, _sz, _sz, _vp, _vp, _vp, _vp]),
+    "fv_vsa_tile_mean": (C.c_int, [_vp, C.c_int, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_int, _vp]),
+    "fv_vsa_coarse": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, C.c_float, _vp]),
+    "fv_vsa_topk": (C.c_int, [_vp, _vp, _sz, _sz, _sz, _vp]),
+    "fv_vsa_tile_qkv": (C.c_int, [_vp, C.c_int, _vp, _vp, _sz, _sz, _sz, _sz, _vp]),
+    "fv_vsa_fine": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_float, _sz, _sz, _vp]),
+    "fv_vsa_combine": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _vp]),
+    "fv_vsa_workspace_bytes": (_sz, [_sz, _sz, _sz, _sz]),
+    "fv_vsa_attention": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp, C.c_int, _vp, _vp, _vp, _vp, _sz, _vp,
+                                   _sz, _sz, _sz, _sz, _sz, C.c_float, _vp]),
+    "fv_block_causal_allows": (C.c_int, [_sz, _sz, _sz, _sz, _sz]),
+    "fv_block_causal_dense_mask": (None, [_sz, _sz, _sz, _sz, _sz, _vp]),
+    "fv_block_causal_for": (C.c_int, [_sz, C.c_longlong, _sz, _vp]),
+    "fv_sp_shard_ranges": (None, [_sz, _sz, _vp]),
 }
 
 _lib = None

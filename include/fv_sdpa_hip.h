@@ -62,6 +62,80 @@ int fv_cast_f32_bf16(const float* x, uint16_t* y, size_t n, void* stream);
 /* bf16 bits -> f32 (exact widening), rt/tensor.rs `to_f32_act`. */
 int fv_cast_bf16_f32(const uint16_t* x, float* y, size_t n, void* stream);
 
+/* ---- Video Sparse Attention (rt/vsa.rs, rt/ops.rs:811-1619) --------------------------
+ * Geometry: 64-token cubes (4x4x4 in t,h,w), TilePlan arrays as rt/vsa.rs:42-109:
+ * slot_src [num_tiles*64] (token of each padded slot, -1 = padding), block_sizes
+ * [num_tiles] (real tokens per tile). Tensors are [bh, seq, dim] in token order or
+ * [bh, num_tiles*64, dim] in tile-slot order ("tile-ordered"). */
+
+/* rt/vsa.rs:34-37 `topk_for`: clamp(ceil((1 - sparsity) * num_tiles), 1, max(num_tiles, 1)). Host. */
+size_t fv_vsa_topk_for(double sparsity, size_t num_tiles);
+/* rt/vsa.rs:62-109 `TilePlan::new`. Host arrays. dims_out = {tiles_t, tiles_h, tiles_w,
+ * seq, padded}; pass NULL arrays to query the dims. Negative return for an empty grid. */
+int fv_vsa_tile_plan(size_t t, size_t h, size_t w, size_t dims_out[5], int32_t* slot_src,
+                     uint32_t* token_slot, int32_t* block_sizes);
+
+/* kernels/core.cu:550-570 `vsa_tile_mean`, kernels/attn3.cu:208-226 `vsa_tile_mean_b16`
+ * (rt/ops.rs:868-872): out[bh, tile, :] = mean of the tile's real tokens, f32 sum in slot
+ * order then / n. x is f32 or bf16 bits [bh, seq, dim]; round16 pools bf16-rounded values
+ * of an f32 x. dim % 4 == 0. */
+int fv_vsa_tile_mean(const void* x, int x_is_bf16, const int32_t* slot_src, const int32_t* block_sizes,
+                     float* out, size_t bh, size_t seq, size_t dim, size_t num_tiles, int round16,
+                     void* stream);
+/* rt/vsa.rs:385-394 (cuBLAS f32 + kernels/core.cu:177-252 `softmax_last` there):
+ * scores[bh, qt, kt] = (qc . kc, summed over d ascending in f32, mul then add) * scale (kept
+ * raw: they drive the selection); coarse[bh, qt, :] = softmax(scores[bh, qt, :]) vc.
+ * coarse may be NULL (scores only). num_tiles <= 4096; coarse needs dim == 128. */
+int fv_vsa_coarse(const float* qc, const float* kc, const float* vc, float* scores, float* coarse,
+                  size_t bh, size_t num_tiles, size_t dim, float scale, void* stream);
+/* kernels/core.cu:584-619 `vsa_topk`, kernels/attn3.cu:279-363 `vsa_topk2` (rt/ops.rs:887-923):
+ * per row of n scores, T = k-th largest key under the order-preserving map of
+ * kernels/core.cu:576-579; out[row, :] = indices with key > T ascending, then key == T
+ * ascending, up to k; zero padded when k > n. Bit-exact. 1 <= n <= 4096. */
+int fv_vsa_topk(const float* scores, uint32_t* out, size_t rows, size_t n, size_t k, void* stream);
+/* kernels/core.cu:1659-1672 `vsa_tile_qkv`, kernels/attn3.cu:230-244 `vsa_tile_qkv_b16`
+ * (rt/ops.rs:1077-1094): token order -> tile-ordered bf16, padding slots zero. dim % 8 == 0. */
+int fv_vsa_tile_qkv(const void* x, int x_is_bf16, const int32_t* slot_src, uint16_t* xt, size_t bh,
+                    size_t seq, size_t padded, size_t dim, void* stream);
+/* kernels/core.cu:1039-1179 `vsa_mma_attn` (+ `_tma`, `_tma2`; rt/ops.rs:1328-1381): for query
+ * tiles [q_base, q_base + q_tiles) of every bh, online softmax over the tiles of
+ * selected[bh, tile, 0..topk) in list order; key columns >= block_sizes[tile] are -inf.
+ * qt/kt/vt tile-ordered bf16; out f32 [bh, q_tiles*64, 128] in tile-slot order. dim == 128. */
+int fv_vsa_fine(const uint16_t* qt, const uint16_t* kt, const uint16_t* vt, const uint32_t* selected,
+                const int32_t* block_sizes, float* out, size_t bh, size_t num_tiles, size_t topk,
+                size_t dim, float scale, size_t q_base, size_t q_tiles, void* stream);
+/* kernels/core.cu:807-835 `vsa_combine` (rt/ops.rs:1592-1601): out[bh, token, :] =
+ * coarse[bh, tile, :] * gate[bh, token, :] + sparse[bh, slot, :] for the real tokens of tiles
+ * [q_base, q_base + q_tiles); gate NULL = 1; gate f32 or bf16 bits. dim == 128. (The H3-only
+ * `round16` variant, kernels/attn3.cu:247-270, is not built.) */
+int fv_vsa_combine(const float* sparse, const float* coarse, const void* gate, int gate_is_bf16,
+                   const int32_t* slot_src, float* out, size_t bh, size_t seq, size_t dim,
+                   size_t num_tiles, size_t q_base, size_t q_tiles, void* stream);
+/* rt/vsa.rs:358-424 `vsa_attention_device` with FineKernel::Mma: tile means -> coarse ->
+ * top-k -> tile permute -> fine -> combine, all on `stream`, using caller-provided scratch
+ * (fv_vsa_workspace_bytes, 256-byte aligned). topk is clamped to [1, num_tiles]. q/k/v (and
+ * gate) are f32 or bf16 bits in token order; out f32 [bh, seq, 128]. selected_out: NULL or
+ * [bh, num_tiles, topk] to receive the block index lists. */
+size_t fv_vsa_workspace_bytes(size_t bh, size_t num_tiles, size_t topk, size_t dim);
+int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf16, const void* gate,
+                     int gate_is_bf16, const int32_t* slot_src, const int32_t* block_sizes, float* out,
+                     void* workspace, size_t workspace_bytes, uint32_t* selected_out, size_t bh,
+                     size_t seq, size_t num_tiles, size_t topk, size_t dim, float scale, void* stream);
+
+/* ---- host-side mask / sharding helpers ------------------------------------------------ */
+/* rt/attn.rs:449-453 `BlockCausal::allows`. */
+int fv_block_causal_allows(size_t block_tokens, size_t window, size_t sink, size_t q, size_t k);
+/* rt/attn.rs:456-466 `BlockCausal::dense_mask`: host [sq, sk], 0 visible / -1e9 masked. */
+void fv_block_causal_dense_mask(size_t block_tokens, size_t window, size_t sink, size_t sq,
+                                size_t sk, float* mask);
+/* rt/attn.rs:630-645 `block_causal_for`: 1 and out3 = {block_tokens, window, 0}, or 0 when the
+ * token window does not cover whole blocks. */
+int fv_block_causal_for(size_t num_frames_per_block, long long local_attn_size, size_t frame_tokens,
+                        size_t out3[3]);
+/* rt/sp.rs:16-28 `shard_ranges`: out[world][2] = (start, len). The library itself never
+ * shards (the full sequence stays on one GPU); kept for callers that do. */
+void fv_sp_shard_ranges(size_t seq, size_t world, size_t* out);
+
 #ifdef __cplusplus
 }
 #endif

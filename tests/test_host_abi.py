@@ -1,0 +1,78 @@
+"""CPU-side checks of the shipped library: it loads, exports every symbol the
+header declares, and its host-side geometry (tile plan, top-k rule, block-causal
+predicate, shard ranges) equals the oracle's restatement of the reference and
+the reference's own known answers. No GPU calls.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from util import ROOT
+
+import fv_sdpa
+from fv_sdpa import _lib
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "fv_sdpa_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(fv_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 20
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert fv_sdpa.lib().fv_sdpa_arch() == b"gfx950"
+    assert fv_sdpa.lib().fv_sdpa_last_error() == b""
+
+
+def test_supported_table():
+    # rt/attn.rs:932-960, d = 128 rows
+    ok = fv_sdpa.sdpa_supported
+    assert ok(1, 40, 38001, 38001, 128) and ok(2, 32, 4097, 1024, 128) and ok(1, 1, 1, 1, 128)
+    for d in (32, 64, 80, 96, 256, 384):
+        assert not ok(1, 8, 1024, 1024, d)
+    assert not ok(1, 8, 0, 1024, 128) and not ok(1, 8, 1024, 0, 128)
+    assert not ok(0, 8, 1024, 1024, 128) and not ok(2, 40000, 64, 64, 128)
+
+
+@pytest.mark.parametrize("grid", [(4, 4, 4), (33, 28, 52), (3, 5, 7), (1, 1, 1), (1, 1, 5), (21, 30, 52), (32, 32, 32)])
+def test_tile_plan_equals_oracle(oracle, grid):
+    got, want = fv_sdpa.TilePlan(grid), oracle.TilePlan(grid)
+    assert got.tiles == want.tiles and got.seq == want.seq and got.padded == want.padded
+    assert np.array_equal(got.slot_src, want.slot_src)
+    assert np.array_equal(got.token_slot, want.token_slot)
+    assert np.array_equal(got.block_sizes.astype(np.uint32), want.block_sizes)
+
+
+def test_tile_plan_known_answers():
+    p = fv_sdpa.TilePlan((1, 1, 5))
+    assert list(p.block_sizes) == [4, 1] and list(p.slot_src[:4]) == [0, 1, 2, 3] and p.slot_src[64] == 4
+    assert (p.slot_src[4:64] == -1).all()
+    assert fv_sdpa.TilePlan((21, 30, 52)).num_tiles == 624
+    with pytest.raises(ValueError):
+        fv_sdpa.TilePlan((4, 0, 4))
+
+
+def test_topk_rule(oracle):
+    for sp, n, want in [(0.8, 819, 164), (0.0, 819, 819), (1.0, 819, 1), (0.9, 10, 1), (0.8, 624, 125), (0.875, 512, 64)]:
+        assert fv_sdpa.topk_for(sp, n) == want == oracle.topk_for(sp, n)
+
+
+def test_block_causal_host_helpers(oracle):
+    for bt, win, sink in [(5, 2, 1), (1, 0, 0), (7, 0, 2), (4, 1, 0), (0, 0, 0), (60, 3, 1)]:
+        assert np.array_equal(fv_sdpa.block_causal_dense_mask(bt, win, sink, 50, 61),
+                              oracle.block_causal_dense_mask(bt, win, sink, 50, 61))
+    for fpb, las, ft in [(3, -1, 1560), (3, 4, 6), (3, 6, 10), (1, 2, 7), (1, -1, 3), (3, 0, 5)]:
+        assert fv_sdpa.block_causal_for(fpb, las, ft) == oracle.block_causal_for(fpb, las, ft)
+    assert fv_sdpa.block_causal_for(3, 4, 6) is None
+    assert fv_sdpa.block_causal_allows(5, 2, 1, 23, 0) and not fv_sdpa.block_causal_allows(5, 2, 1, 23, 5)
+
+
+def test_shard_ranges(oracle):
+    assert fv_sdpa.shard_ranges(10, 2) == [(0, 5), (5, 5)]
+    assert fv_sdpa.shard_ranges(11, 2) == [(0, 6), (6, 5)]
+    assert fv_sdpa.shard_ranges(32760, 8) == oracle.shard_ranges(32760, 8)
