@@ -34,7 +34,8 @@ FV_DEV void lds_dma16(unsigned lds_base, const void* gptr) {
         "global_load_lds_dwordx4 %1, off"
         :
         : "s"(lds_base), "v"(gptr)
-        : "memory", "m0");
+        : "memory");   // m0 is a reserved scratch register: the compiler sets it right before
+                       // each of its own uses and keeps nothing live in it across statements
 }
 
 // Workgroup barrier without the memory fences of __syncthreads() (a fence

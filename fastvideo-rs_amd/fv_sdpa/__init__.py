@@ -5,3 +5,4 @@ torch is used only for device memory and streams.
 from ._lib import FvDeclined, FvError, LIB_PATH, build, lib  # noqa: F401
 from .ops import *  # noqa: F401,F403
 from .vsa import *  # noqa: F401,F403
+from .sdpa import *  # noqa: F401,F403

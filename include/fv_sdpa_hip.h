@@ -62,6 +62,56 @@ int fv_cast_f32_bf16(const float* x, uint16_t* y, size_t n, void* stream);
 /* bf16 bits -> f32 (exact widening), rt/tensor.rs `to_f32_act`. */
 int fv_cast_bf16_f32(const uint16_t* x, float* y, size_t n, void* stream);
 
+/* rt/sdpa.rs:328-342 `sdpa_composed` on the device: out = softmax(scale * q k^T + mask) v,
+ * f32 operands [bh, s, d] and f32 out; mask NULL, or additive [sq, sk] shared by every bh
+ * (mask_per_bh == 0), or [bh, sq, sk] (mask_per_bh != 0). The path for masked calls and for
+ * shapes the fused kernels decline (it replaces the reference's cuBLAS-materialised and
+ * scalar-flash fallbacks, rt/attn.rs:59-88, 748-865). 1 <= d <= 256. */
+int fv_sdpa_composed_f32(const float* q, const float* k, const float* v, const float* mask,
+                         int mask_per_bh, float* out, size_t bh, size_t sq, size_t sk, size_t d,
+                         float scale, void* stream);
+
+/* ---- the one entry: rt::sdpa::sdpa(q, k, v, &Plan) (rt/sdpa.rs:141-164), flattened ------- */
+typedef struct fv_tensor {
+    void* data;        /* device pointer, contiguous row-major */
+    int dtype;         /* 0 = f32, 1 = bf16 bits (rt/tensor.rs:28-32) */
+    int rank;
+    size_t shape[8];
+} fv_tensor;
+
+enum {
+    FV_PLAN_DENSE = 0,        /* Plan::dense / Plan::masked / .fp8_first() (rt/sdpa.rs:56-88) */
+    FV_PLAN_COMPOSED = 1,     /* Plan::composed (rt/sdpa.rs:93-98) */
+    FV_PLAN_BLOCK_CAUSAL = 2, /* Plan::block_causal (rt/sdpa.rs:104-109) */
+    FV_PLAN_VDN_WINDOW = 3,   /* Plan::vdn_window (rt/sdpa.rs:114-119): refused, kernel not built */
+    FV_PLAN_KV_WINDOW = 4     /* Plan::kv_window / kv_window_with (rt/sdpa.rs:125-137) */
+};
+
+typedef struct fv_plan {
+    int kind;
+    int has_scale;            /* 0: scale = 1/sqrt(d) */
+    float scale;
+    const fv_tensor* mask;    /* additive [.., sq, sk] for DENSE / COMPOSED, else NULL */
+    int fp8_first;            /* accepted and ignored: this library is bf16 only */
+    size_t block_tokens, window, sink;   /* BLOCK_CAUSAL */
+    int kv_flash;             /* KV_WINDOW: -1 = FASTVIDEO_WAN_CAUSAL_FLASH, 0 composed f32, 1 dense route */
+} fv_plan;
+
+/* Runs the plan on `stream`. q [b,h,sq,d], k/v [b,h,sk,d], f32 or bf16. On FV_OK `out` describes
+ * a NEW device buffer owned by the caller (free with fv_rt_free or hipFree): bf16 under bf16
+ * activations (FASTVIDEO_BF16_ACT, default on), else f32 (rt/sdpa.rs:184-214). Temporaries are
+ * allocated stream-ordered. Errors return a negative code; fv_sdpa_last_error() holds the
+ * reference's message ("sdpa expects BHSD", "sdpa: every kernel of the route declined", ...). */
+int fv_rt_sdpa(const fv_tensor* q, const fv_tensor* k, const fv_tensor* v, const fv_plan* plan,
+               fv_tensor* out, void* stream);
+int fv_rt_free(void* p, void* stream);
+/* rt/tensor.rs `with_bf16_act`: per-thread override of FASTVIDEO_BF16_ACT; v < 0 clears it. */
+void fv_rt_set_bf16_activations(int v);
+int fv_rt_bf16_activations(void);
+/* rt/stats.rs:27-72 analogue: {fused dense launches, block-causal launches, composed launches,
+ * cast launches, dense masks materialised} since the library was loaded. */
+void fv_rt_stats(uint64_t out5[5]);
+
 /* ---- Video Sparse Attention (rt/vsa.rs, rt/ops.rs:811-1619) --------------------------
  * Geometry: 64-token cubes (4x4x4 in t,h,w), TilePlan arrays as rt/vsa.rs:42-109:
  * slot_src [num_tiles*64] (token of each padded slot, -1 = padding), block_sizes

@@ -1,0 +1,185 @@
+"""The `sdpa(q, k, v, &Plan)` entry on the device, read like the reference's own unit
+tests (crates/fastvideo-cudarc/src/rt/sdpa.rs:508-575, rt/attn.rs:905-1002): plan
+equivalences, refusals, the block-causal fallback, dtype rules under bf16 activations —
+plus parity of the device composed path against the fp32 oracle.
+"""
+import numpy as np
+import pytest
+
+from util import announce, assert_parity, metrics, qkv, randn
+from test_oracle_sdpa import sin_tensor
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fv():
+    import torch
+
+    assert torch.cuda.is_available()
+    import fv_sdpa
+
+    fv_sdpa.lib()
+    return fv_sdpa
+
+
+def dev(x):
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def host(t):
+    import torch
+
+    torch.cuda.synchronize()
+    return t.float().cpu().numpy()
+
+
+def test_dense_plans_without_a_fused_kernel_are_the_composed_reference(fv, oracle):
+    # rt/sdpa.rs:522-542: 1x2x5x7x8 (d = 8: the fused kernel declines, every plan is composed)
+    announce("rt plans == composed, 1x2x5x7x8")
+    b, h, sq, sk, d = 1, 2, 5, 7, 8
+    q = sin_tensor(b * h * sq * d, 0.37, (b, h, sq, d))
+    k = sin_tensor(b * h * sk * d, 0.71, (b, h, sk, d))
+    v = sin_tensor(b * h * sk * d, 1.13, (b, h, sk, d))
+    P = fv.Plan
+    with fv.with_bf16_act(False):
+        want = host(fv.sdpa(dev(q), dev(k), dev(v), P.composed(None, None)))
+        for plan in (P.dense(None), P.dense(None).fp8_first(), P.masked(None, None), P.composed(None, None),
+                     P.kv_window_with(True), P.kv_window_with(False)):
+            got = fv.sdpa(dev(q), dev(k), dev(v), plan)
+            assert got.dtype.is_floating_point and got.element_size() == 4
+            assert np.array_equal(host(got), want)
+        scaled = host(fv.sdpa(dev(q), dev(k), dev(v), P.dense(0.5)))
+        assert not np.array_equal(scaled, want)
+    ref = oracle.sdpa_composed(q.reshape(h, sq, d), k.reshape(h, sk, d), v.reshape(h, sk, d))
+    assert np.abs(want.reshape(h, sq, d) - ref).max() < 2e-6
+
+
+def test_non_bhsd_operands_are_refused(fv):
+    q = dev(np.zeros((2, 4), np.float32))
+    with pytest.raises(fv.TensorError, match="BHSD"):
+        fv.sdpa(q, q, q, fv.Plan.dense(None))
+
+
+def test_vdn_window_is_refused_not_misrun(fv):
+    q = dev(np.zeros((1, 1, 4, 128), np.float32))
+    with pytest.raises(fv.TensorError, match="vdn_window"):
+        fv.sdpa(q, q, q, fv.Plan.vdn_window(None))
+
+
+def test_block_causal_fallback_matches_the_masked_composed_sdpa(fv, oracle):
+    # rt/attn.rs:905-930: S = 24, d = 8, BlockCausal{5, 2, 1}
+    announce("rt block-causal fallback 1x2x24x8")
+    b, h, s, d = 1, 2, 24, 8
+    q = sin_tensor(b * h * s * d, 0.37, (b, h, s, d))
+    k = sin_tensor(b * h * s * d, 0.71, (b, h, s, d))
+    v = sin_tensor(b * h * s * d, 1.13, (b, h, s, d))
+    spec = fv.BlockCausal(5, 2, 1)
+    before = fv.rt_stats()
+    with fv.with_bf16_act(False):
+        got = host(fv.sdpa(dev(q), dev(k), dev(v), fv.Plan.block_causal(None, spec)))
+        mask = dev(spec.dense_mask(s, s).reshape(1, 1, s, s))
+        want = host(fv.sdpa(dev(q), dev(k), dev(v), fv.Plan.masked(None, mask)))
+        dense = host(fv.sdpa(dev(q), dev(k), dev(v), fv.Plan.dense(None)))
+    assert np.array_equal(got, want)
+    assert not np.array_equal(got[0, 0, 0], dense[0, 0, 0])
+    after = fv.rt_stats()
+    assert after["masks"] == before["masks"] + 1 and after["composed"] == before["composed"] + 3
+    ref = oracle.sdpa_composed(q.reshape(h, s, d), k.reshape(h, s, d), v.reshape(h, s, d),
+                               mask=oracle.block_causal_dense_mask(5, 2, 1, s, s))
+    assert np.abs(got.reshape(h, s, d) - ref).max() < 2e-6
+
+
+def test_dense_bf16_act_psnr_vs_f32(fv):
+    # rt/attn.rs:986-1002
+    import torch
+
+    q = dev(((np.arange(24, dtype=np.float32) * np.float32(0.13)) - np.float32(0.8)).reshape(1, 2, 3, 4))
+    with fv.with_bf16_act(False):
+        f32_out = fv.sdpa(q, q, q, fv.Plan.dense(None))
+    with fv.with_bf16_act(True):
+        bf16_out = fv.sdpa(q, q, q, fv.Plan.dense(None))
+    assert f32_out.dtype == torch.float32 and bf16_out.dtype == torch.bfloat16
+    a, r = host(bf16_out).astype(np.float64), host(f32_out).astype(np.float64)
+    rng_ = 2.0 * max(np.abs(r).max(), 1.0)
+    psnr = 10 * np.log10(rng_ * rng_ / np.mean((a - r) ** 2))
+    assert psnr >= 35.0
+
+
+@pytest.mark.parametrize("act16", [False, True])
+@pytest.mark.parametrize("f32_in", [False, True])
+def test_dense_plan_reaches_the_fused_kernel(fv, oracle, act16, f32_in):
+    import torch
+
+    b, h, sq, sk, d = 1, 3, 200, 300, 128
+    announce(f"rt dense fused act16={act16} f32_in={f32_in}")
+    q, k, v = qkv(300, b * h, sq, sk, d)
+    shape = lambda x, s: x.reshape(b, h, s, d)
+    mk = (lambda x: dev(x)) if f32_in else (lambda x: dev(x).to(torch.bfloat16))
+    tq, tk, tv = mk(shape(q, sq)), mk(shape(k, sk)), mk(shape(v, sk))
+    before = fv.rt_stats()
+    with fv.with_bf16_act(act16):
+        got = fv.sdpa(tq, tk, tv, fv.Plan.dense(None))
+    after = fv.rt_stats()
+    assert after["fused"] == before["fused"] + 1 and after["composed"] == before["composed"]
+    assert got.dtype == (torch.bfloat16 if act16 else torch.float32) and tuple(got.shape) == (b, h, sq, d)
+    # bit-identical to the direct kernel call (G/kernels.rs "default dispatch" check)
+    direct = fv.sdpa_dense_bf16(dev(q).to(torch.bfloat16), dev(k).to(torch.bfloat16), dev(v).to(torch.bfloat16),
+                                out_bf16=act16)
+    torch.cuda.synchronize()
+    assert torch.equal(got.reshape(b * h, sq, d), direct)
+    assert_parity(host(got).reshape(b * h, sq, d), oracle.sdpa_composed(q, k, v), "rt_dense_fused",
+                  max_abs=2e-2 if act16 else 1e-2)
+
+
+def test_block_causal_and_kv_window_plans_at_d128(fv, oracle):
+    import torch
+
+    b, h, s, d, bt = 1, 2, 384, 128, 96
+    announce("rt block-causal / kv-window d128")
+    q, k, v = qkv(400, b * h, s, s, d)
+    t4 = lambda x: dev(x.reshape(b, h, s, d)).to(torch.bfloat16)
+    before = fv.rt_stats()
+    with fv.with_bf16_act(False):
+        got = fv.sdpa(t4(q), t4(k), t4(v), fv.Plan.block_causal(None, fv.BlockCausal(bt, 0, 0)))
+        kvw = fv.sdpa(t4(q)[:, :, :100].contiguous(), t4(k), t4(v), fv.Plan.kv_window())
+        kvc = fv.sdpa(t4(q)[:, :, :100].contiguous(), t4(k), t4(v), fv.Plan.kv_window_with(False))
+    after = fv.rt_stats()
+    assert after["causal"] == before["causal"] + 1 and after["masks"] == before["masks"]
+    want = oracle.sdpa_composed(q, k, v, mask=oracle.block_causal_dense_mask(bt, 0, 0, s, s))
+    assert_parity(host(got).reshape(b * h, s, d), want, "rt_block_causal")
+    wantw = oracle.sdpa_composed(q[:, :100], k, v)
+    assert_parity(host(kvw).reshape(b * h, 100, d), wantw, "rt_kv_window_flash")
+    assert np.abs(host(kvc).reshape(b * h, 100, d) - wantw).max() < 1e-5
+
+
+@pytest.mark.parametrize("bh,sq,sk,d,mask_kind", [(2, 5, 7, 8, None), (3, 33, 300, 64, "shared"), (2, 40, 257, 128, "per_bh"),
+                                                  (1, 3, 1000, 256, None), (2, 64, 64, 128, "shared"), (1, 2, 1, 128, None)])
+def test_composed_kernel_vs_oracle(fv, oracle, bh, sq, sk, d, mask_kind):
+    import ctypes
+    import torch
+
+    announce(f"composed f32 bh={bh} sq={sq} sk={sk} d={d} mask={mask_kind}")
+    q, k, v = qkv(500 + sq, bh, sq, sk, d, round_bf16=False)
+    mask = None
+    if mask_kind == "shared":
+        mask = oracle.block_causal_dense_mask(max(sk // 5, 1), 0, 1, sq, sk)
+    elif mask_kind == "per_bh":
+        mask = (randn(7, (bh, sq, sk)) * 2).astype(np.float32)
+    tq, tk, tv = dev(q), dev(k), dev(v)
+    tm = dev(mask) if mask is not None else None
+    out = torch.empty((bh, sq, d), device="cuda", dtype=torch.float32)
+    scale = 1.0 / np.sqrt(d)
+    rc = fv.lib().fv_sdpa_composed_f32(tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), tm.data_ptr() if tm is not None else None,
+                                       int(mask_kind == "per_bh"), out.data_ptr(), bh, sq, sk, d, scale,
+                                       torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, fv.lib().fv_sdpa_last_error()
+    if mask_kind == "per_bh":
+        want = np.stack([oracle.sdpa_composed(q[i:i + 1], k[i:i + 1], v[i:i + 1], mask=mask[i])[0] for i in range(bh)])
+    else:
+        want = oracle.sdpa_composed(q, k, v, mask=mask)
+    m = metrics(host(out), want)
+    print(m)
+    assert m["max_abs"] < 2e-5
