@@ -50,12 +50,71 @@ FV_DEV void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// LDS-DMA with a wave-uniform 64-bit base (SGPR pair) + per-lane byte offset.
+FV_DEV void lds_dma16_s(unsigned lds_base, const void* sbase_in, unsigned voff) {
+    // pin the base to an SGPR pair even where the compiler's divergence analysis
+    // (branches on the wave index) would otherwise place it in VGPRs
+    const unsigned long long a = (unsigned long long)sbase_in;
+    // (readfirstlane returns int: widen through unsigned, or a low half with bit 31 set
+    // would sign-extend over the high half)
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)a);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(a >> 32));
+    const unsigned long long sbase = ((unsigned long long)hi << 32) | (unsigned long long)lo;
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %2"
+        :
+        : "s"(lds_base), "v"(voff), "s"(sbase)
+        : "memory");
+}
+
+// Per-lane source offsets of the tile loads, computed once per kernel: with NW
+// waves sharing a 64-row tile a wave issues ITER = 16 / NW instructions of 4 rows
+// each; instruction `it` of wave w covers rows (w*ITER + it)*4 .. +3, lane i
+// fetching the 16 B chunk that belongs at position i%16 of row + i/16.
+template <int NW>
+struct TileDma {
+    static constexpr int ITER = 16 / NW;
+    unsigned koff[ITER];   // byte offset from the tile's first row, K swizzle
+    unsigned voff[ITER];   // same, V swizzle
+    FV_DEV void init(int wave, int lane) {
+        const int p = lane & 15;
+#pragma unroll
+        for (int it = 0; it < ITER; it++) {
+            const int r = (wave * ITER + it) * 4 + (lane >> 4);
+            koff[it] = r * kRowBytes + ((p ^ (r & 15)) << 4);
+            voff[it] = r * kRowBytes + ((p ^ ((r & 3) << 2)) << 4);
+        }
+    }
+    // tile_base (wave-uniform) points at the tile's first row. Rows >= rows_valid
+    // re-read the last valid row: the caller masks their scores to -inf, so their
+    // content only has to be finite data the tensor already holds.
+    template <bool IS_V>
+    FV_DEV void issue(lds_u8* buf, const uint16_t* tile_base, int rows_valid, int wave) const {
+        const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 4 * kRowBytes);
+        if (rows_valid >= kTileRows) {
+#pragma unroll
+            for (int it = 0; it < ITER; it++)
+                lds_dma16_s(base + it * 4 * kRowBytes, tile_base, IS_V ? voff[it] : koff[it]);
+        } else {
+#pragma unroll
+            for (int it = 0; it < ITER; it++) {
+                const unsigned off = IS_V ? voff[it] : koff[it];
+                const int over = max(0, (int)(off >> 8) - (rows_valid - 1));
+                lds_dma16_s(base + it * 4 * kRowBytes, tile_base, off - over * kRowBytes);
+            }
+        }
+    }
+};
+
 // Issue the asynchronous loads of one 64 x 128 bf16 tile whose rows are
 // contiguous in global memory (256 B apart). NW waves share the tile, 4 rows
 // per wave instruction. Rows >= rows_valid re-read the last valid row (the
 // caller masks their scores to -inf, so their content only has to be finite
 // data the tensor already holds). Completion is tracked by vmcnt: 16 / NW
-// instructions per wave and tile.
+// instructions per wave and tile. This is the general (tail-safe) form; full
+// tiles go through TileDma::issue.
 template <int NW, bool IS_V>
 FV_DEV void tile_load_async(lds_u8* buf, const uint16_t* g, int rows_valid, int wave, int lane) {
     constexpr int ITER = 16 / NW;
@@ -174,6 +233,66 @@ FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 
             o[db] = mfma32(__builtin_bit_cast(bf16x8, a), pb[t], o[db]);
         }
     }
+}
+
+// One MFMA phase with a deep, explicit LDS prefetch: O^T += V^T P^T of the
+// previous tile (groups 0-7, if DO_PV) followed by S^T = K Q^T of the current
+// one (groups 8-15). A group is 2 operand fragments (8 VGPRs) feeding 2 MFMAs on
+// different accumulators. kAhead (2-3, bounded by the 256-VGPR budget) groups are always in flight ahead of the group
+// being multiplied, so an MFMA waits on a read issued kAhead x 64 cycles of
+// matrix-pipe time earlier instead of on LDS latency plus the 64 B/clk per-SIMD
+// LDS return path. sched_barrier keeps the compiler from re-serialising reads
+// behind MFMAs.
+template <bool DO_PV, int kAhead>
+FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& rb,
+                       const bf16x8 (&pb)[4], f32x16 (&o)[4], const bf16x8 (&qf)[8],
+                       f32x16 (&s)[2], long long* ts = nullptr) {
+    constexpr int G0 = DO_PV ? 0 : 8;
+    bf16x8 f[16][2];
+    auto issue = [&](int g) {
+        if (g < 8) {          // V^T fragments: key group t = g/2, d blocks 2*(g%2), 2*(g%2)+1
+#pragma unroll
+            for (int x = 0; x < 2; x++) {
+                const int t = g >> 1, db = 2 * (g & 1) + x;
+                const int a0 = (rb.v ^ (db << 6)) + (16 * t) * kRowBytes;
+                s16x8 a;
+                a.lo = lds_read_tr16_b64(vb + a0);
+                a.hi = lds_read_tr16_b64(vb + a0 + 8 * kRowBytes);
+                f[g][x] = __builtin_bit_cast(bf16x8, a);
+            }
+        } else {              // K fragments: d chunk dk = g-8, key blocks 0 and 1
+#pragma unroll
+            for (int x = 0; x < 2; x++)
+                f[g][x] = lds_read_b128(kb + (rb.k ^ ((g - 8) << 5)) + x * 32 * kRowBytes);
+        }
+    };
+    auto run = [&](int g) {
+        if (g < 8) {
+#pragma unroll
+            for (int x = 0; x < 2; x++) {
+                const int t = g >> 1, db = 2 * (g & 1) + x;
+                o[db] = mfma32(f[g][x], pb[t], o[db]);
+            }
+        } else {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                                 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int x = 0; x < 2; x++)   // S is born at dk == 0, not before the PV part
+                s[x] = mfma32(f[g][x], qf[g - 8], g == 8 ? zero : s[x]);
+        }
+    };
+#pragma unroll
+    for (int g = G0; g < G0 + kAhead && g < 16; g++) issue(g);
+    if (ts) ts[0] = __builtin_readcyclecounter();
+#pragma unroll
+    for (int g = G0; g < 16; g++) {
+        if (g + kAhead < 16) issue(g + kAhead);
+        __builtin_amdgcn_sched_barrier(0);
+        run(g);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ts && (g == 3 || g == 7 || g == 11)) ts[1 + g / 4] = __builtin_readcyclecounter();
+    }
+    if (ts) ts[4] = __builtin_readcyclecounter();
 }
 
 // Q^T fragments for the wave's 32 queries: rows row0 + lane%32 of a row-major

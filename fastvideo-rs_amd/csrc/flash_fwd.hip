@@ -25,7 +25,9 @@
 //   * workgroup ids are remapped so that the workgroups resident on one XCD
 //     walk consecutive query tiles of the same head (their K/V stream hits
 //     that XCD's L2).
-#include "fv_common.h"
+#include <stdlib.h>
+
+#include "attn_core.h"
 #include "fv_internal.h"
 
 namespace fv {
@@ -39,7 +41,6 @@ constexpr int kKBytes = kBN * kKStride;
 constexpr int kVBytes = kBN * kVStride;
 constexpr int kStageBytes = kKBytes + kVBytes;
 constexpr int kFlashLdsBytes = 2 * kStageBytes;
-constexpr float kRescaleLog2 = 6.0f;
 
 
 template <bool CAUSAL>
@@ -291,25 +292,289 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const FlashParams p) {
     }
 }
 
+
+// ---- ping-pong variant ------------------------------------------------------------------
+// One workgroup = 8 waves = 256 queries; waves 0-3 (group 0) and 4-7 (group 1)
+// share the SIMDs pairwise and run half an iteration apart: while one group is
+// in its MFMA phase (O += P V of the previous tile, S = K Q^T of the current
+// one) the other is in its VALU phase (softmax of its current tile), separated
+// by workgroup barriers, so each SIMD's matrix pipe and vector ALU are busy at
+// the same time by construction instead of by chance.
+//
+// Time is counted in slots (one phase each). Group 0 runs MFMA(j) in slot 2j and
+// VALU(j) in slot 2j+1; group 1 is one slot behind. K and V tiles rotate
+// through kStages LDS buffers each (swizzled, LDS-DMA fed): at even slot 2m
+// every wave issues its share of K(m+2) and V(m+1), which are first read in
+// slot 2m+4 — four slots (~2 us) of load latency are hidden.
+constexpr int kPpBM = 256;
+constexpr int kStages = 3;
+constexpr int kPpLdsBytes = 2 * kStages * kTileBytes;   // K[3], V[3] = 96 KB
+
+template <bool CAUSAL>
+__global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    lds_u8* smem = (lds_u8*)smem_raw;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int grp = wave >> 2;
+    const int h = lane >> 5, c32 = lane & 31;
+    const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (work >= p.total) return;
+    const int bh = work / p.nqt;
+    const int qt = CAUSAL ? (p.nqt - 1 - work % p.nqt) : (work % p.nqt);
+    const int q0 = qt * kPpBM;
+    const int sq = p.sq, sk = p.sk;
+    const int qlen = min(kPpBM, sq - q0);
+    const float sl2 = p.sl2;
+    const float NEG = neg_inf();
+
+    const uint16_t* Qh = p.q + ((size_t)bh * sq + q0) * kD;
+    const uint16_t* Kh = p.k + (size_t)bh * sk * kD;
+    const uint16_t* Vh = p.v + (size_t)bh * sk * kD;
+
+    const int nkt = (sk + kBN - 1) / kBN;
+    int ns = 0, mlo = 0, ne = nkt;
+    int hi_q = 0, lo_q = 0, sink_tok = 0;
+    if constexpr (CAUSAL) {
+        const int ft = p.ft, win = p.win;
+        const int fq_lo = q0 / ft, fq_hi = (q0 + qlen - 1) / ft;
+        const int hi_tok = (int)min((long)sk, (long)(fq_hi + 1) * ft);
+        const int lo_tok = min(hi_tok, win > 0 ? max(0, fq_lo - win + 1) * ft : 0);
+        sink_tok = (int)min((long)sk, (long)p.sink * ft);
+        const int sink_tiles = (sink_tok + kBN - 1) / kBN;
+        mlo = lo_tok / kBN;
+        const int mhi = max((hi_tok + kBN - 1) / kBN, sink_tiles);
+        ns = min(sink_tiles, mlo);
+        ne = ns + (mhi - mlo);
+        const int tq = (q0 + wave * 32 + c32) / ft;
+        hi_q = (int)min((long)0x7fffffff, (long)(tq + 1) * ft);
+        lo_q = win > 0 ? max(0, tq - win + 1) * ft : 0;
+    }
+    auto tile_of = [&](int e) -> int {
+        if constexpr (CAUSAL) return e < ns ? e : mlo + (e - ns);
+        else return e;
+    };
+    auto kbuf = [&](int e) -> lds_u8* { return smem + (e % kStages) * kTileBytes; };
+    auto vbuf = [&](int e) -> lds_u8* { return smem + (kStages + e % kStages) * kTileBytes; };
+
+    TileDma<8> dma;
+    dma.init(wave, lane);
+    // returns the number of DMA instructions this wave issued (0 or 2)
+    auto issue_k = [&](int e) -> int {
+#ifdef FV_X_NODMA
+        if (e > 2) return 0;
+#endif
+        if (e >= ne) return 0;
+        const int kv0 = tile_of(e) * kBN;
+        dma.issue<false>(kbuf(e), Kh + (size_t)kv0 * kD, sk - kv0, wave);
+        return 2;
+    };
+    auto issue_v = [&](int e) -> int {
+#ifdef FV_X_NODMA
+        if (e > 2) return 0;
+#endif
+        if (e >= ne) return 0;
+        const int kv0 = tile_of(e) * kBN;
+        dma.issue<true>(vbuf(e), Vh + (size_t)kv0 * kD, sk - kv0, wave);
+        return 2;
+    };
+    // the loads issued one even slot ago must have landed; those just issued may fly on
+    auto wait_older = [&](int just_issued) {
+        if (just_issued == 4) wait_vmcnt<4>();
+        else if (just_issued == 2) wait_vmcnt<2>();
+        else wait_vmcnt<0>();
+    };
+
+#ifdef FV_PROF
+    long long* prof = (long long*)p.out_f32 + (size_t)wave * 512;
+    int pi = 0;
+    const bool prof_on = blockIdx.x == 64 && lane == 0;
+    if (prof_on) prof[511] = __builtin_amdgcn_s_getreg((4) | (0 << 6) | (31 << 11));   // HW_ID
+#ifdef FV_PROF2
+#define FV_TS() do {} while (0)
+#else
+#define FV_TS() do { if (prof_on && pi < 500) prof[pi++] = __builtin_readcyclecounter(); } while (0)
+#endif
+#else
+#define FV_TS() do {} while (0)
+#endif
+    issue_k(0);
+    issue_k(1);
+    issue_v(0);
+    bf16x8 qf[8];
+    {
+        const int row = wave * 32 + c32;
+        load_q_frags(Qh, row, row < qlen, lane, qf);   // drains vmcnt: the three tiles have landed too
+    }
+    const TileReadBases rb = tile_read_bases(lane);
+
+    f32x16 o[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[db][i] = 0.f;
+    SoftmaxState st;
+    st.init();
+    f32x16 s[2];
+    bf16x8 pb[4];     // P of the previous tile; zero before the first one
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int x = 0; x < 8; x++) pb[t][x] = (__bf16)0.0f;
+
+#ifdef FV_X_G0ONLY
+    if (grp == 1) return;
+#endif
+#ifdef FV_X_G1ONLY
+    if (grp == 0) return;
+#endif
+    block_barrier();                 // K(0), K(1), V(0) resident
+    int flying = 0;                  // DMA instructions this wave issued in the current even slot
+    if (grp == 1) {                  // slot 0: group 1 only feeds the pipeline
+        flying = issue_k(2) + issue_v(1);
+        __builtin_amdgcn_sched_barrier(0);
+        block_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+#pragma unroll 1
+    for (int j = 0; j < ne; j++) {
+        // ---- MFMA phase: group 0 in slot 2j, group 1 in slot 2j+1 ----
+        if (grp == 0) flying = issue_k(j + 2) + issue_v(j + 1);
+        __builtin_amdgcn_s_setprio(1);
+        constexpr int kAhead = CAUSAL ? 2 : 3;   // LDS prefetch depth the register budget allows
+        // P starts as zero, so the first pass adds 0 * V(0) (finite, resident) and needs no special case
+        mfma_phase<true, kAhead>(vbuf(j > 0 ? j - 1 : 0), kbuf(j), rb, pb, o, qf, s);
+        __builtin_amdgcn_s_setprio(0);
+        FV_TS();
+        if (grp == 1) wait_older(flying);
+        __builtin_amdgcn_sched_barrier(0);
+        block_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        FV_TS();
+        // ---- VALU phase: group 0 in slot 2j+1, group 1 in slot 2j+2 ----
+        if (grp == 1) flying = issue_k(j + 3) + issue_v(j + 2);
+        const int kv0 = tile_of(j) * kBN;
+        if (kv0 + kBN > sk) {
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
+                    if (key >= sk) s[b][i] = NEG;
+                }
+        }
+        if constexpr (CAUSAL) {
+            const int kend = min(kv0 + kBN, sk);
+            const bool lane_all = (kend <= hi_q && kv0 >= lo_q) || kend <= sink_tok;
+            if (__builtin_amdgcn_ballot_w64(!lane_all) != 0) {
+#pragma unroll
+                for (int b = 0; b < 2; b++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
+                        const bool vis = (key < hi_q && key >= lo_q) || key < sink_tok;
+                        if (!vis) s[b][i] = NEG;
+                    }
+            }
+        }
+#ifdef FV_X_NOSOFTMAX
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                f32x8 f;
+#pragma unroll
+                for (int x = 0; x < 8; x++) f[x] = s[b][8 * t + x];
+                pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
+            }
+        st.l_acc += s[0][0];
+#elif defined(FV_X_G1_NOSOFTMAX)
+        if (grp == 0) softmax_tile(s, st, o, sl2, pb);
+        else {
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                f32x8 f;
+#pragma unroll
+                for (int x = 0; x < 8; x++) f[x] = s[b][8 * t + x];
+                pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
+            }
+        st.l_acc += s[0][0];
+        }
+#else
+        softmax_tile(s, st, o, sl2, pb);
+#endif
+        FV_TS();
+        if (grp == 0) wait_older(flying);
+        if (grp == 0 || j + 1 < ne) {
+            __builtin_amdgcn_sched_barrier(0);
+            block_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        FV_TS();
+    }
+    if (ne > 0) {
+        // O += P V of the last tile (its V landed before the last barrier both groups passed)
+        pv_tile(vbuf(ne - 1), rb.v, pb, o);
+    }
+
+    const float l_tot = pair_sum(st.l_acc);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int row = wave * 32 + c32;
+    if (row < qlen) {
+        const size_t base = ((size_t)bh * sq + q0 + row) * kD;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d0 = 32 * db + 8 * g + 4 * h;
+                f32x4 r;
+#pragma unroll
+                for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
+                if (p.out_is_bf16) {
+                    const bf16x4 rb4 = __builtin_convertvector(r, bf16x4);
+                    *reinterpret_cast<bf16x4*>(p.out_bf16 + base + d0) = rb4;
+                } else {
+                    *reinterpret_cast<f32x4*>(p.out_f32 + base + d0) = r;
+                }
+            }
+    }
+}
+
 }  // namespace fv
 
 // ---- host launchers -------------------------------------------------------------
 
+extern "C" int fv_internal_flash_block_m(void) {
+    static const int bm = [] {
+        const char* e = getenv("FV_FLASH_KERNEL");
+        return (e && e[0] == 'v' && e[1] == '1') ? fv::kBM : fv::kPpBM;
+    }();
+    return bm;
+}
+
 extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal,
                                                hipStream_t stream) {
-    static bool attr_done[2] = {false, false};
-    const void* fn = causal ? (const void*)fv::flash_fwd_d128<true>
-                            : (const void*)fv::flash_fwd_d128<false>;
-    if (!attr_done[causal]) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           fv::kFlashLdsBytes);
+    const bool pp = fv_internal_flash_block_m() == fv::kPpBM;
+    static bool attr_done[4] = {false, false, false, false};
+    const void* fn = pp ? (causal ? (const void*)fv::flash_fwd_pp_d128<true> : (const void*)fv::flash_fwd_pp_d128<false>)
+                        : (causal ? (const void*)fv::flash_fwd_d128<true> : (const void*)fv::flash_fwd_d128<false>);
+    const int lds = pp ? fv::kPpLdsBytes : fv::kFlashLdsBytes;
+    const int idx = (pp ? 2 : 0) + causal;
+    if (!attr_done[idx]) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
-        attr_done[causal] = true;
+        attr_done[idx] = true;
     }
-    const dim3 grid(p->per_xcd * 8), block(256);
-    if (causal)
-        hipLaunchKernelGGL(fv::flash_fwd_d128<true>, grid, block, fv::kFlashLdsBytes, stream, *p);
-    else
-        hipLaunchKernelGGL(fv::flash_fwd_d128<false>, grid, block, fv::kFlashLdsBytes, stream, *p);
+    const dim3 grid(p->per_xcd * 8), block(pp ? 512 : 256);
+    if (pp) {
+        if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp_d128<true>, grid, block, lds, stream, *p);
+        else hipLaunchKernelGGL(fv::flash_fwd_pp_d128<false>, grid, block, lds, stream, *p);
+    } else {
+        if (causal) hipLaunchKernelGGL(fv::flash_fwd_d128<true>, grid, block, lds, stream, *p);
+        else hipLaunchKernelGGL(fv::flash_fwd_d128<false>, grid, block, lds, stream, *p);
+    }
     return hipGetLastError();
 }

@@ -11,6 +11,10 @@
 #include "fv_internal.h"
 
 static thread_local std::string g_last_error;
+#ifdef FV_PROF
+void* g_fv_prof_buf = nullptr;
+extern "C" void* fv_prof_buf(void) { return g_fv_prof_buf; }
+#endif
 
 int fv_fail_hip(hipError_t e, const char* what) {
     char buf[256];
@@ -63,12 +67,21 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
     p.k = k;
     p.v = v;
     p.out_f32 = out_is_bf16 ? nullptr : (float*)out;
+#ifdef FV_PROF
+    {
+        static void* dbg = nullptr;
+        if (!dbg) { (void)hipMalloc(&dbg, 8 * 512 * 8); (void)hipMemset(dbg, 0, 8 * 512 * 8); }
+        p.out_f32 = (float*)dbg;
+        ::g_fv_prof_buf = dbg;
+    }
+#endif
     p.out_bf16 = out_is_bf16 ? (uint16_t*)out : nullptr;
     p.out_is_bf16 = out_is_bf16 ? 1 : 0;
     p.sq = (int)sq;
     p.sk = (int)sk;
     p.sl2 = scale * 1.4426950408889634f;
-    p.nqt = (int)((sq + 127) / 128);
+    const size_t bm = (size_t)fv_internal_flash_block_m();
+    p.nqt = (int)((sq + bm - 1) / bm);
     const size_t total = bh * (size_t)p.nqt;
     if (total > (size_t)INT_MAX / 2) return decline("sdpa: too many query tiles for one launch");
     p.total = (int)total;
