@@ -243,10 +243,10 @@ FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 
 // matrix-pipe time earlier instead of on LDS latency plus the 64 B/clk per-SIMD
 // LDS return path. sched_barrier keeps the compiler from re-serialising reads
 // behind MFMAs.
-template <bool DO_PV, int kAhead>
+template <bool DO_PV, int kAhead, class Hook>
 FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& rb,
                        const bf16x8 (&pb)[4], f32x16 (&o)[4], const bf16x8 (&qf)[8],
-                       f32x16 (&s)[2], long long* ts = nullptr) {
+                       f32x16 (&s)[2], Hook&& hook) {
     constexpr int G0 = DO_PV ? 0 : 8;
     bf16x8 f[16][2];
     auto issue = [&](int g) {
@@ -283,16 +283,14 @@ FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& 
     };
 #pragma unroll
     for (int g = G0; g < G0 + kAhead && g < 16; g++) issue(g);
-    if (ts) ts[0] = __builtin_readcyclecounter();
 #pragma unroll
     for (int g = G0; g < 16; g++) {
         if (g + kAhead < 16) issue(g + kAhead);
         __builtin_amdgcn_sched_barrier(0);
         run(g);
         __builtin_amdgcn_sched_barrier(0);
-        if (ts && (g == 3 || g == 7 || g == 11)) ts[1 + g / 4] = __builtin_readcyclecounter();
+        hook(g);   // side work (tile DMA issue) that rides under the matrix pipe
     }
-    if (ts) ts[4] = __builtin_readcyclecounter();
 }
 
 // Q^T fragments for the wave's 32 queries: rows row0 + lane%32 of a row-major

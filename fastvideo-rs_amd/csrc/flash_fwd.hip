@@ -303,9 +303,15 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const FlashParams p) {
 //
 // Time is counted in slots (one phase each). Group 0 runs MFMA(j) in slot 2j and
 // VALU(j) in slot 2j+1; group 1 is one slot behind. K and V tiles rotate
-// through kStages LDS buffers each (swizzled, LDS-DMA fed): at even slot 2m
-// every wave issues its share of K(m+2) and V(m+1), which are first read in
-// slot 2m+4 — four slots (~2 us) of load latency are hidden.
+// through 3 LDS buffers each (swizzled, LDS-DMA fed). Every wave issues its
+// share (2 + 2 instructions) of K(j+2) and V(j+1) from inside its MFMA phase j,
+// where the address arithmetic and the issue ride under the matrix pipe, and
+// waits for them (vmcnt) at the end of its MFMA phase j+1; both tiles are first
+// read in MFMA phase j+2 / j+1's successor, at least three slots after issue.
+// The buffers they overwrite held K(j-1) and V(j-2), last read in MFMA phase
+// j-1 of either group, which ended at least one barrier before any wave's
+// phase j began. Past the last tile the loads re-fetch the last tile into a
+// buffer nobody reads, which keeps the issue and wait counts constant.
 constexpr int kPpBM = 256;
 constexpr int kStages = 3;
 constexpr int kPpLdsBytes = 2 * kStages * kTileBytes;   // K[3], V[3] = 96 KB
@@ -315,7 +321,8 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     lds_u8* smem = (lds_u8*)smem_raw;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: branches on it stay scalar
     const int grp = wave >> 2;
     const int h = lane >> 5, c32 = lane & 31;
     const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
@@ -350,57 +357,31 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
         hi_q = (int)min((long)0x7fffffff, (long)(tq + 1) * ft);
         lo_q = win > 0 ? max(0, tq - win + 1) * ft : 0;
     }
+    if (ne <= 0) return;   // cannot happen for sk >= 1 (the walk always holds the query's own block)
+    // key-tile index of walk position e; positions past the end repeat the last tile
     auto tile_of = [&](int e) -> int {
+        e = min(e, ne - 1);
         if constexpr (CAUSAL) return e < ns ? e : mlo + (e - ns);
         else return e;
     };
-    auto kbuf = [&](int e) -> lds_u8* { return smem + (e % kStages) * kTileBytes; };
-    auto vbuf = [&](int e) -> lds_u8* { return smem + (kStages + e % kStages) * kTileBytes; };
+    auto kbuf = [&](int st) -> lds_u8* { return smem + st * kTileBytes; };
+    auto vbuf = [&](int st) -> lds_u8* { return smem + (kStages + st) * kTileBytes; };
+    auto next_stage = [](int st) -> int { return st == kStages - 1 ? 0 : st + 1; };
 
     TileDma<8> dma;
     dma.init(wave, lane);
-    // returns the number of DMA instructions this wave issued (0 or 2)
-    auto issue_k = [&](int e) -> int {
-#ifdef FV_X_NODMA
-        if (e > 2) return 0;
-#endif
-        if (e >= ne) return 0;
+    auto issue_k = [&](int e, int st) {
         const int kv0 = tile_of(e) * kBN;
-        dma.issue<false>(kbuf(e), Kh + (size_t)kv0 * kD, sk - kv0, wave);
-        return 2;
+        dma.issue<false>(kbuf(st), Kh + (size_t)kv0 * kD, sk - kv0, wave);
     };
-    auto issue_v = [&](int e) -> int {
-#ifdef FV_X_NODMA
-        if (e > 2) return 0;
-#endif
-        if (e >= ne) return 0;
+    auto issue_v = [&](int e, int st) {
         const int kv0 = tile_of(e) * kBN;
-        dma.issue<true>(vbuf(e), Vh + (size_t)kv0 * kD, sk - kv0, wave);
-        return 2;
-    };
-    // the loads issued one even slot ago must have landed; those just issued may fly on
-    auto wait_older = [&](int just_issued) {
-        if (just_issued == 4) wait_vmcnt<4>();
-        else if (just_issued == 2) wait_vmcnt<2>();
-        else wait_vmcnt<0>();
+        dma.issue<true>(vbuf(st), Vh + (size_t)kv0 * kD, sk - kv0, wave);
     };
 
-#ifdef FV_PROF
-    long long* prof = (long long*)p.out_f32 + (size_t)wave * 512;
-    int pi = 0;
-    const bool prof_on = blockIdx.x == 64 && lane == 0;
-    if (prof_on) prof[511] = __builtin_amdgcn_s_getreg((4) | (0 << 6) | (31 << 11));   // HW_ID
-#ifdef FV_PROF2
-#define FV_TS() do {} while (0)
-#else
-#define FV_TS() do { if (prof_on && pi < 500) prof[pi++] = __builtin_readcyclecounter(); } while (0)
-#endif
-#else
-#define FV_TS() do {} while (0)
-#endif
-    issue_k(0);
-    issue_k(1);
-    issue_v(0);
+    issue_k(0, 0);
+    issue_k(1, 1);
+    issue_v(0, 0);
     bf16x8 qf[8];
     {
         const int row = wave * 32 + c32;
@@ -422,38 +403,28 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
 #pragma unroll
         for (int x = 0; x < 8; x++) pb[t][x] = (__bf16)0.0f;
 
-#ifdef FV_X_G0ONLY
-    if (grp == 1) return;
-#endif
-#ifdef FV_X_G1ONLY
-    if (grp == 0) return;
-#endif
     block_barrier();                 // K(0), K(1), V(0) resident
-    int flying = 0;                  // DMA instructions this wave issued in the current even slot
-    if (grp == 1) {                  // slot 0: group 1 only feeds the pipeline
-        flying = issue_k(2) + issue_v(1);
-        __builtin_amdgcn_sched_barrier(0);
-        block_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-    }
+    if (grp == 1) block_barrier();   // group 1 idles through slot 0
 
+    // LDS stages: K(j) in sk_cur, K(j+2) goes to sk_ld = stage of j-1; V(j-1) in sv_prev, V(j+1)
+    // goes to the stage after V(j)
+    int sk_cur = 0, sk_ld = 2, sv_prev = 0, sv_ld = 1;
 #pragma unroll 1
     for (int j = 0; j < ne; j++) {
         // ---- MFMA phase: group 0 in slot 2j, group 1 in slot 2j+1 ----
-        if (grp == 0) flying = issue_k(j + 2) + issue_v(j + 1);
         __builtin_amdgcn_s_setprio(1);
         constexpr int kAhead = CAUSAL ? 2 : 3;   // LDS prefetch depth the register budget allows
         // P starts as zero, so the first pass adds 0 * V(0) (finite, resident) and needs no special case
-        mfma_phase<true, kAhead>(vbuf(j > 0 ? j - 1 : 0), kbuf(j), rb, pb, o, qf, s);
+        mfma_phase<true, kAhead>(vbuf(sv_prev), kbuf(sk_cur), rb, pb, o, qf, s, [&](int g) {
+            if (g == 1) issue_k(j + 2, sk_ld);
+            if (g == 4) issue_v(j + 1, sv_ld);
+        });
         __builtin_amdgcn_s_setprio(0);
-        FV_TS();
-        if (grp == 1) wait_older(flying);
+        wait_vmcnt<4>();             // this wave's loads of the previous phase have landed
         __builtin_amdgcn_sched_barrier(0);
         block_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        FV_TS();
         // ---- VALU phase: group 0 in slot 2j+1, group 1 in slot 2j+2 ----
-        if (grp == 1) flying = issue_k(j + 3) + issue_v(j + 2);
         const int kv0 = tile_of(j) * kBN;
         if (kv0 + kBN > sk) {
 #pragma unroll
@@ -478,47 +449,23 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
                     }
             }
         }
-#ifdef FV_X_NOSOFTMAX
-#pragma unroll
-        for (int b = 0; b < 2; b++)
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                f32x8 f;
-#pragma unroll
-                for (int x = 0; x < 8; x++) f[x] = s[b][8 * t + x];
-                pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
-            }
-        st.l_acc += s[0][0];
-#elif defined(FV_X_G1_NOSOFTMAX)
-        if (grp == 0) softmax_tile(s, st, o, sl2, pb);
-        else {
-#pragma unroll
-        for (int b = 0; b < 2; b++)
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                f32x8 f;
-#pragma unroll
-                for (int x = 0; x < 8; x++) f[x] = s[b][8 * t + x];
-                pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
-            }
-        st.l_acc += s[0][0];
-        }
-#else
         softmax_tile(s, st, o, sl2, pb);
-#endif
-        FV_TS();
-        if (grp == 0) wait_older(flying);
+        // P and the row sum must be complete before the barrier: without this the
+        // compiler sinks the exponentials past it, into the matrix phase
+        asm volatile("" ::"v"(pb[0]), "v"(pb[1]), "v"(pb[2]), "v"(pb[3]), "v"(st.l_acc));
+        sv_prev = j > 0 ? next_stage(sv_prev) : 0;   // V(j) lives in stage j % 3
+        sv_ld = next_stage(sv_ld);
+        sk_ld = sk_cur;
+        sk_cur = next_stage(sk_cur);
         if (grp == 0 || j + 1 < ne) {
             __builtin_amdgcn_sched_barrier(0);
             block_barrier();
             __builtin_amdgcn_sched_barrier(0);
         }
-        FV_TS();
     }
-    if (ne > 0) {
-        // O += P V of the last tile (its V landed before the last barrier both groups passed)
-        pv_tile(vbuf(ne - 1), rb.v, pb, o);
-    }
+    // O += P V of the last tile (its V landed before the last barrier both groups passed)
+    pv_tile(vbuf(sv_prev), rb.v, pb, o);
+    wait_vmcnt<0>();   // the redundant tail loads must not outlive the workgroup's LDS
 
     const float l_tot = pair_sum(st.l_acc);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
