@@ -87,6 +87,32 @@ struct TileDma {
             voff[it] = r * kRowBytes + ((p ^ ((r & 3) << 2)) << 4);
         }
     }
+    // A tile load prepared ahead of its issue: everything the DMA instructions need,
+    // so that issuing them from inside a matrix phase costs 3 instructions each.
+    struct Prepared {
+        unsigned long long base;   // wave-uniform global address of the tile's first row
+        unsigned lds;              // wave-uniform LDS byte address of this wave's first row
+        unsigned off[ITER];        // per-lane byte offsets (tail rows clamped)
+    };
+    template <bool IS_V>
+    FV_DEV Prepared prepare(lds_u8* buf, const uint16_t* tile_base, int rows_valid, int wave) const {
+        Prepared d;
+        d.base = (unsigned long long)tile_base;
+        d.lds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 4 * kRowBytes);
+#pragma unroll
+        for (int it = 0; it < ITER; it++) d.off[it] = IS_V ? voff[it] : koff[it];
+        if (rows_valid < kTileRows) {
+#pragma unroll
+            for (int it = 0; it < ITER; it++) {
+                const int over = max(0, (int)(d.off[it] >> 8) - (rows_valid - 1));
+                d.off[it] -= over * kRowBytes;
+            }
+        }
+        return d;
+    }
+    static FV_DEV void issue_prepared(const Prepared& d, int it) {
+        lds_dma16_s(d.lds + it * 4 * kRowBytes, (const void*)d.base, d.off[it]);
+    }
     // tile_base (wave-uniform) points at the tile's first row. Rows >= rows_valid
     // re-read the last valid row: the caller masks their scores to -inf, so their
     // content only has to be finite data the tensor already holds.

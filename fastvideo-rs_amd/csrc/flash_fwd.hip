@@ -334,6 +334,13 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
     const int qlen = min(kPpBM, sq - q0);
     const float sl2 = p.sl2;
     const float NEG = neg_inf();
+    // Fetch the epilogue's arguments now. Left to the compiler, their scalar loads sit
+    // right before the main loop, still pending at its head, and a pending scalar load
+    // (out-of-order return) turns every LDS wait count in the loop into a full drain.
+    float* out_f32 = p.out_f32;
+    uint16_t* out_bf16 = p.out_bf16;
+    int out_is_bf16 = p.out_is_bf16;
+    asm volatile("" : "+s"(out_f32), "+s"(out_bf16), "+s"(out_is_bf16));
 
     const uint16_t* Qh = p.q + ((size_t)bh * sq + q0) * kD;
     const uint16_t* Kh = p.k + (size_t)bh * sk * kD;
@@ -403,6 +410,17 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
 #pragma unroll
         for (int x = 0; x < 8; x++) pb[t][x] = (__bf16)0.0f;
 
+    // the loads a matrix phase issues are prepared (addresses, tail clamp) one VALU phase earlier
+    auto prep_k = [&](int e, int st) {
+        const int kv0 = tile_of(e) * kBN;
+        return dma.prepare<false>(kbuf(st), Kh + (size_t)kv0 * kD, sk - kv0, wave);
+    };
+    auto prep_v = [&](int e, int st) {
+        const int kv0 = tile_of(e) * kBN;
+        return dma.prepare<true>(vbuf(st), Vh + (size_t)kv0 * kD, sk - kv0, wave);
+    };
+    TileDma<8>::Prepared dk = prep_k(2, 2), dv = prep_v(1, 1);
+
     block_barrier();                 // K(0), K(1), V(0) resident
     if (grp == 1) block_barrier();   // group 1 idles through slot 0
 
@@ -416,8 +434,10 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
         constexpr int kAhead = CAUSAL ? 2 : 3;   // LDS prefetch depth the register budget allows
         // P starts as zero, so the first pass adds 0 * V(0) (finite, resident) and needs no special case
         mfma_phase<true, kAhead>(vbuf(sv_prev), kbuf(sk_cur), rb, pb, o, qf, s, [&](int g) {
-            if (g == 1) issue_k(j + 2, sk_ld);
-            if (g == 4) issue_v(j + 1, sv_ld);
+            if (g == 1) TileDma<8>::issue_prepared(dk, 0);
+            if (g == 2) TileDma<8>::issue_prepared(dk, 1);
+            if (g == 4) TileDma<8>::issue_prepared(dv, 0);
+            if (g == 5) TileDma<8>::issue_prepared(dv, 1);
         });
         __builtin_amdgcn_s_setprio(0);
         wait_vmcnt<4>();             // this wave's loads of the previous phase have landed
@@ -457,6 +477,8 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
         sv_ld = next_stage(sv_ld);
         sk_ld = sk_cur;
         sk_cur = next_stage(sk_cur);
+        dk = prep_k(j + 3, sk_ld);   // for matrix phase j+1: K(j+3), V(j+2)
+        dv = prep_v(j + 2, sv_ld);
         if (grp == 0 || j + 1 < ne) {
             __builtin_amdgcn_sched_barrier(0);
             block_barrier();
@@ -480,11 +502,11 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
                 f32x4 r;
 #pragma unroll
                 for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
-                if (p.out_is_bf16) {
+                if (out_is_bf16) {
                     const bf16x4 rb4 = __builtin_convertvector(r, bf16x4);
-                    *reinterpret_cast<bf16x4*>(p.out_bf16 + base + d0) = rb4;
+                    *reinterpret_cast<bf16x4*>(out_bf16 + base + d0) = rb4;
                 } else {
-                    *reinterpret_cast<f32x4*>(p.out_f32 + base + d0) = r;
+                    *reinterpret_cast<f32x4*>(out_f32 + base + d0) = r;
                 }
             }
     }
