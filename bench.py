@@ -23,6 +23,9 @@ sys.path.insert(0, os.path.join(ROOT, "fastvideo-rs_amd"))
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the flash kernel at the headline workload, from two counter runs
+# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from a plain 1 GiB copy in the same runs).
+MEASURED_TRAFFIC_BYTES = {"self": 1.0065e9}
 
 WORKLOADS = {
     # name: (H, Sq, Sk, causal block_tokens or 0, description)
@@ -89,6 +92,9 @@ def main():
     ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
+    ap.add_argument("--copy-calibration-mib", type=int, default=0,
+                    help="also launch one plain device copy of this many MiB (known HBM traffic, to scale "
+                         "profiler byte counters); not part of the timed region")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the full sequence on ONE GPU (no sharding, no collectives); "
@@ -126,6 +132,13 @@ def main():
         if rc != 0:
             raise RuntimeError(f"kernel rc={rc}: {lib.fv_sdpa_last_error().decode()}")
 
+    if args.copy_calibration_mib > 0:
+        src = torch.empty(args.copy_calibration_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)   # one elementwise copy kernel: reads and writes exactly this many bytes
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -167,8 +180,9 @@ def main():
                    "dense_equivalent_flops": flops_dense_equiv},
         "pct_of_bf16_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                     "kernel": "flash_fwd_d128<causal>" if bt else "flash_fwd_d128",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.out_bf16 else None,
+                     "kernel": "fv::flash_fwd_pp_d128<true>" if bt else "fv::flash_fwd_pp_d128<false>",
                      "avg_kernel_ms": round(avg_kernel_ms, 4), "median_kernel_ms": round(kern_ms[len(kern_ms) // 2], 4),
                      "min_hbm_bytes": bytes_min,
                      "hbm_frac_at_min_traffic": round(bytes_min / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
