@@ -8,8 +8,8 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny) are for the design notes;
-the driver's line is the default `self`.
+Other workloads (--workload cross|causal|causal3|c5|tiny|vsa624|vsa512) are for the
+design notes; the driver's line is the default `self`.
 """
 import argparse
 import json
@@ -37,6 +37,82 @@ WORKLOADS = {
     "c5cross": (40, 75600, 512, 0, "Wan2.1-14B 720p cross-attention, H=40 Sq=75600 Sk=512"),
     "tiny": (12, 320, 320, 0, "tiny Wan-1.3B-shaped self-attention, H=12 S=320 d=128"),
 }
+
+
+VSA_WORKLOADS = {
+    # name: (H, grid, sparsity, description)
+    "vsa624": (12, (21, 30, 52), 0.8, "VSA, Wan 480p latent grid (21,30,52): 624 tiles, top-k 125, H=12 d=128"),
+    "vsa512": (12, (32, 32, 32), 0.875, "VSA, 512 full 4x4x4 cubes (32768 tokens), top-k 64, H=12 d=128"),
+}
+
+
+def bench_vsa(args):
+    """Whole VSA op (tile means, coarse scores + top-k, tile pass, block-sparse fine
+    kernel, combine) plus each stage alone; FLOPs credited are the fine stage's
+    4*(bh*nb*64)*(topk*64)*d, the reference's convention (gpucheck kernels/attn3.rs:747)."""
+    import torch
+
+    import fv_sdpa
+    from fv_sdpa import vsa as V
+
+    fv_sdpa.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    h, grid, sparsity, desc = VSA_WORKLOADS[args.workload]
+    d = 128
+    ctx = V.VsaCtx(grid, sparsity, device=dev)
+    nb, topk, seq = ctx.num_tiles, ctx.topk, ctx.seq
+    g = torch.Generator(device=dev).manual_seed(20241)
+    q, k, v, gate = (torch.randn((h, seq, d), generator=g, device=dev).to(torch.bfloat16) for _ in range(4))
+    scale = 1.0 / d ** 0.5
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        t0 = time.perf_counter()
+        for a, b in evs:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        ms = sorted(a.elapsed_time(b) for a, b in evs)
+        return wall, sum(ms) / len(ms), ms[len(ms) // 2]
+
+    wall, avg_ms, med_ms = timed(lambda: V.vsa_attention_device(q, k, v, gate, ctx, scale), args.steps, args.warmup)
+    # stages alone, on the same operands
+    qc, kc, vc = (V.vsa_tile_mean(x, ctx) for x in (q, k, v))
+    scores, coarse = V.vsa_coarse(qc, kc, vc, scale)
+    sel = V.vsa_topk(scores, topk)
+    qt, kt, vt = (V.vsa_tile_qkv(x, ctx) for x in (q, k, v))
+    sparse = V.vsa_fine(qt, kt, vt, sel, ctx, scale)
+    out = torch.empty((h, seq, d), device=dev, dtype=torch.float32)
+    stages = {
+        "tile_mean_x3": timed(lambda: [V.vsa_tile_mean(x, ctx) for x in (q, k, v)], 10, 2)[2],
+        "coarse_scores_softmax_pv": timed(lambda: V.vsa_coarse(qc, kc, vc, scale), 10, 2)[2],
+        "topk": timed(lambda: V.vsa_topk(scores, topk), 10, 2)[2],
+        "tile_qkv_x3": timed(lambda: [V.vsa_tile_qkv(x, ctx) for x in (q, k, v)], 10, 2)[2],
+        "fine": timed(lambda: V.vsa_fine(qt, kt, vt, sel, ctx, scale), 10, 2)[2],
+        "combine": timed(lambda: V.vsa_combine(sparse, coarse, gate, ctx, out=out), 10, 2)[2],
+    }
+    flops = 4.0 * (h * nb * 64) * (topk * 64) * d
+    fine_tflops = flops / (stages["fine"] * 1e-3) / 1e12
+    rec = {
+        "metric": f"VSA TFLOP/s ({args.workload}, fine-stage FLOPs over whole-op time)",
+        "value": round(flops / (wall * 1e-3) / 1e12, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": desc, "H": h, "grid": list(grid), "tiles": nb, "topk": topk, "seq": seq, "d": d,
+                   "inputs": "bf16 q/k/v/gate", "flops_per_call": flops},
+        "whole_op_avg_ms": round(avg_ms, 4), "whole_op_median_ms": round(med_ms, 4),
+        "stages_median_ms": {k2: round(v2, 4) for k2, v2 in stages.items()},
+        "roofline": {"bound": "mfma", "achieved": round(fine_tflops, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(fine_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::vsa_fine_kernel",
+                     "avg_kernel_ms": round(stages["fine"], 4)},
+    }
+    print(json.dumps(rec), flush=True)
 
 
 def visible_pairs(sq, sk, bt):
@@ -89,7 +165,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -108,6 +184,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
+    if args.workload in VSA_WORKLOADS:
+        bench_vsa(args)
+        return
     fv_sdpa.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)

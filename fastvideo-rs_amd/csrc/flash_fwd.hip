@@ -5,7 +5,7 @@
 // attn::device_mma_sdpa / device_mma_sdpa_causal (rt/attn.rs:225-421, 652-730).
 //
 // Schedule (not a translation of the CUDA one):
-//   * one workgroup = 4 waves = 128 queries of one (batch, head); each wave
+//   * one workgroup = 8 waves = 256 queries of one (batch, head); each wave
 //     owns 32 queries and walks the keys in tiles of 64;
 //   * the wave computes S^T = K Q^T with v_mfma_f32_32x32x16_bf16: K rows come
 //     from LDS as the A operand, Q^T stays in registers as the B operand for
@@ -20,298 +20,39 @@
 //     accumulator is rescaled only when some row's max grew by more than
 //     2^kRescaleLog2 since the last rescale; the final O / l is exact for any
 //     such choice because P and l always share the same reference max;
-//   * K/V tiles are prefetched global -> registers -> LDS (two LDS stages, one
-//     barrier per tile);
+//   * waves 0-3 (group 0) and 4-7 (group 1) share the SIMDs pairwise and run
+//     half an iteration apart: while one group is in its MFMA phase (O += P V
+//     of the previous tile, S = K Q^T of the current one, operands prefetched
+//     from LDS a fixed number of MFMAs ahead) the other is in its VALU phase
+//     (softmax of its current tile), separated by workgroup barriers, so each
+//     SIMD's matrix pipe and vector ALU are busy at the same time by
+//     construction. Interleaving the two instruction kinds inside one wave
+//     loses on this hardware: a wave issues in order, so its VALU work stalls
+//     behind every MFMA that waits for the matrix pipe;
+//   * K/V tiles go global -> LDS directly (global_load_lds_dwordx4) into
+//     XOR-swizzled unpadded tiles, three stages each;
 //   * workgroup ids are remapped so that the workgroups resident on one XCD
 //     walk consecutive query tiles of the same head (their K/V stream hits
 //     that XCD's L2).
-#include <stdlib.h>
-
+//
+// Time is counted in slots (one phase each). Group 0 runs MFMA(j) in slot 2j and
+// VALU(j) in slot 2j+1; group 1 is one slot behind. Every wave issues its
+// share (2 + 2 instructions) of K(j+2) and V(j+1) from inside its MFMA phase j,
+// from descriptors (addresses, tail clamp) prepared in the VALU phase before,
+// and waits for them (vmcnt) at the end of its MFMA phase j+1; both tiles are
+// first read at least three slots after issue. The buffers they overwrite held
+// K(j-1) and V(j-2), last read in MFMA phase j-1 of either group, which ended
+// at least one barrier before any wave's phase j began. Past the last tile the
+// loads re-fetch the last tile into a buffer nobody reads, which keeps the
+// issue and wait counts constant.
 #include "attn_core.h"
 #include "fv_internal.h"
 
 namespace fv {
 
 constexpr int kD = 128;          // head dim
-constexpr int kBM = 128;         // queries per workgroup
 constexpr int kBN = 64;          // keys per tile
-constexpr int kKStride = 272;    // bytes per K row in LDS (256 + 16 pad)
-constexpr int kVStride = 320;    // bytes per V row in LDS (256 + 64 pad)
-constexpr int kKBytes = kBN * kKStride;
-constexpr int kVBytes = kBN * kVStride;
-constexpr int kStageBytes = kKBytes + kVBytes;
-constexpr int kFlashLdsBytes = 2 * kStageBytes;
 
-
-template <bool CAUSAL>
-__global__ __launch_bounds__(256, 2) void flash_fwd_d128(const FlashParams p) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    lds_u8* smem = (lds_u8*)smem_raw;
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int h = lane >> 5, c32 = lane & 31;
-
-    // XCD-aware work assignment: workgroup ids go round-robin over the 8 XCDs,
-    // so id%8 picks the XCD and id/8 the position in that XCD's contiguous
-    // range of (head, query tile) work items.
-    const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-    if (work >= p.total) return;
-    const int bh = work / p.nqt;
-    // causal: heaviest (latest) query tiles first
-    const int qt = CAUSAL ? (p.nqt - 1 - work % p.nqt) : (work % p.nqt);
-    const int q0 = qt * kBM;
-    const int sq = p.sq, sk = p.sk;
-    const int qlen = min(kBM, sq - q0);
-    const float sl2 = p.sl2;
-    const float NEG = neg_inf();
-
-    const uint16_t* Qh = p.q + ((size_t)bh * sq + q0) * kD;
-    const uint16_t* Kh = p.k + (size_t)bh * sk * kD;
-    const uint16_t* Vh = p.v + (size_t)bh * sk * kD;
-
-    // ---- key-tile walk: [0, ns) then [mlo, mlo + ne - ns) --------------------
-    const int nkt = (sk + kBN - 1) / kBN;
-    int ns = 0, mlo = 0, ne = nkt;
-    int hi_q = 0, lo_q = 0, sink_tok = 0;   // this lane's visible key range
-    if constexpr (CAUSAL) {
-        const int ft = p.ft, win = p.win;
-        const int fq_lo = q0 / ft, fq_hi = (q0 + qlen - 1) / ft;
-        const int hi_tok = (int)min((long)sk, (long)(fq_hi + 1) * ft);
-        const int lo_tok = min(hi_tok, win > 0 ? max(0, fq_lo - win + 1) * ft : 0);
-        sink_tok = (int)min((long)sk, (long)p.sink * ft);
-        const int sink_tiles = (sink_tok + kBN - 1) / kBN;
-        mlo = lo_tok / kBN;
-        // sink blocks are visible to every query, also to those before them
-        const int mhi = max((hi_tok + kBN - 1) / kBN, sink_tiles);
-        ns = min(sink_tiles, mlo);
-        ne = ns + (mhi - mlo);
-        const int tq = (q0 + wave * 32 + c32) / ft;
-        hi_q = (int)min((long)0x7fffffff, (long)(tq + 1) * ft);
-        lo_q = win > 0 ? max(0, tq - win + 1) * ft : 0;
-    }
-    auto tile_of = [&](int e) -> int {
-        if constexpr (CAUSAL) return e < ns ? e : mlo + (e - ns);
-        else return e;
-    };
-
-    // ---- Q^T fragments (B operand), resident for the whole kernel ------------
-    bf16x8 qf[8];
-    {
-        const int row = wave * 32 + c32;
-        const bool ok = row < qlen;
-        const uint16_t* src = Qh + (size_t)row * kD + 8 * h;
-#pragma unroll
-        for (int dk = 0; dk < 8; dk++) {
-            u32x4 t = {0u, 0u, 0u, 0u};
-            if (ok) t = *reinterpret_cast<const u32x4*>(src + 16 * dk);
-            qf[dk] = __builtin_bit_cast(bf16x8, t);
-        }
-    }
-
-    // ---- global -> register staging of one K/V tile --------------------------
-    // 64 rows x 16 chunks of 16 B per tensor; thread t takes chunks t + 256 i.
-    u32x4 gk[4], gv[4];
-    const int ld_row = tid >> 4, ld_col = tid & 15;
-    auto load_tile = [&](int kt) {
-        const int kv0 = kt * kBN;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int row = kv0 + ld_row + 16 * i;
-            u32x4 a = {0u, 0u, 0u, 0u}, b = {0u, 0u, 0u, 0u};
-            if (row < sk) {
-                const size_t off = (size_t)row * kD + ld_col * 8;
-                a = *reinterpret_cast<const u32x4*>(Kh + off);
-                b = *reinterpret_cast<const u32x4*>(Vh + off);
-            }
-            gk[i] = a;
-            gv[i] = b;
-        }
-    };
-    auto store_tile = [&](int stage) {
-        lds_u8* kb = smem + stage * kStageBytes;
-        lds_u8* vb = kb + kKBytes;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int row = ld_row + 16 * i;
-            lds_write_b128(kb + row * kKStride + ld_col * 16, gk[i]);
-            lds_write_b128(vb + row * kVStride + ld_col * 16, gv[i]);
-        }
-    };
-
-    // per-lane LDS read offsets
-    const int k_rd = c32 * kKStride + h * 16;                       // + kb*32*kKStride + dk*32
-    const int b16 = lane >> 4, i16 = lane & 15;
-    const int v_rd = (4 * h + (i16 >> 2)) * kVStride + (16 * (b16 & 1) + 4 * (i16 & 3)) * 2;
-    // + (16 t + 8 g) * kVStride + db * 64
-
-    f32x16 o[4];
-#pragma unroll
-    for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) o[db][i] = 0.f;
-    float m_run = NEG;     // running row max (raw scores)
-    float ms_used = 0.f;   // m_used * sl2, the exponent offset P and l refer to
-    float m_used = NEG;
-    float l_acc = 0.f;     // this lane's share of the row sum
-
-    if (ne > 0) {
-        load_tile(tile_of(0));
-        store_tile(0);
-    }
-    __syncthreads();
-
-#pragma unroll 1
-    for (int j = 0; j < ne; j++) {
-        const int kt = tile_of(j);
-        const int kv0 = kt * kBN;
-        const int stage = j & 1;
-        if (j + 1 < ne) load_tile(tile_of(j + 1));
-
-        const lds_u8* kb = smem + stage * kStageBytes;
-        const lds_u8* vb = kb + kKBytes;
-
-        // S^T = K Q^T : two 32-key blocks
-        f32x16 s[2];
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) s[b][i] = 0.f;
-#pragma unroll
-            for (int dk = 0; dk < 8; dk++) {
-                const bf16x8 a = lds_read_b128(kb + k_rd + b * 32 * kKStride + dk * 32);
-                s[b] = mfma32(a, qf[dk], s[b]);
-            }
-        }
-
-        // key of s[b][i]: kv0 + 32 b + 8 (i/4) + 4 h + i%4
-        if (kv0 + kBN > sk) {
-#pragma unroll
-            for (int b = 0; b < 2; b++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
-                    if (key >= sk) s[b][i] = NEG;
-                }
-        }
-        if constexpr (CAUSAL) {
-            const int kend = min(kv0 + kBN, sk);
-            const bool lane_all = (kend <= hi_q && kv0 >= lo_q) || kend <= sink_tok;
-            if (__builtin_amdgcn_ballot_w64(!lane_all) != 0) {
-#pragma unroll
-                for (int b = 0; b < 2; b++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
-                        const bool vis = (key < hi_q && key >= lo_q) || key < sink_tok;
-                        if (!vis) s[b][i] = NEG;
-                    }
-            }
-        }
-
-        // row max over this lane's 32 keys, then the other half's
-        float mx = s[0][0];
-#pragma unroll
-        for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s[0][i]);
-#pragma unroll
-        for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s[1][i]);
-        mx = pair_max(mx);
-        m_run = __builtin_fmaxf(m_run, mx);
-
-        // rescale when some row's max outgrew the offset in use
-        const bool need = (m_run * sl2 - ms_used > kRescaleLog2) || (m_used == NEG && m_run != NEG);
-        if (__builtin_amdgcn_ballot_w64(need) != 0) {
-            const float ms_new = (m_run == NEG) ? 0.f : m_run * sl2;
-            const float alpha = (m_used == NEG) ? 0.f : fast_exp2(ms_used - ms_new);
-            l_acc *= alpha;
-#pragma unroll
-            for (int db = 0; db < 4; db++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) o[db][i] *= alpha;
-            m_used = m_run;
-            ms_used = ms_new;
-        }
-
-        // P = 2^(s*sl2 - ms_used), row-sum share, bf16 pack
-        bf16x8 pb[4];
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-            f32x16 e;
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                e[i] = fast_exp2(__builtin_fmaf(s[b][i], sl2, -ms_used));
-                l_acc += e[i];
-            }
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                f32x8 f;
-#pragma unroll
-                for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
-                pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
-            }
-        }
-
-        // O^T += V^T P^T
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-#pragma unroll
-            for (int db = 0; db < 4; db++) {
-                const s16x4 lo = lds_read_tr16_b64(vb + v_rd + (16 * t) * kVStride + db * 64);
-                const s16x4 hi = lds_read_tr16_b64(vb + v_rd + (16 * t + 8) * kVStride + db * 64);
-                s16x8 a;
-                a.lo = lo;
-                a.hi = hi;
-                o[db] = mfma32(__builtin_bit_cast(bf16x8, a), pb[t], o[db]);
-            }
-        }
-
-        if (j + 1 < ne) store_tile(stage ^ 1);
-        __syncthreads();
-    }
-
-    // ---- epilogue: O / l, written row-major [query][d] -------------------------
-    const float l_tot = pair_sum(l_acc);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    const int row = wave * 32 + c32;
-    if (row < qlen) {
-        const size_t base = ((size_t)bh * sq + q0 + row) * kD;
-#pragma unroll
-        for (int db = 0; db < 4; db++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int d0 = 32 * db + 8 * g + 4 * h;
-                f32x4 r;
-#pragma unroll
-                for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
-                if (p.out_is_bf16) {
-                    const bf16x4 rb = __builtin_convertvector(r, bf16x4);
-                    *reinterpret_cast<bf16x4*>(p.out_bf16 + base + d0) = rb;
-                } else {
-                    *reinterpret_cast<f32x4*>(p.out_f32 + base + d0) = r;
-                }
-            }
-    }
-}
-
-
-// ---- ping-pong variant ------------------------------------------------------------------
-// One workgroup = 8 waves = 256 queries; waves 0-3 (group 0) and 4-7 (group 1)
-// share the SIMDs pairwise and run half an iteration apart: while one group is
-// in its MFMA phase (O += P V of the previous tile, S = K Q^T of the current
-// one) the other is in its VALU phase (softmax of its current tile), separated
-// by workgroup barriers, so each SIMD's matrix pipe and vector ALU are busy at
-// the same time by construction instead of by chance.
-//
-// Time is counted in slots (one phase each). Group 0 runs MFMA(j) in slot 2j and
-// VALU(j) in slot 2j+1; group 1 is one slot behind. K and V tiles rotate
-// through 3 LDS buffers each (swizzled, LDS-DMA fed). Every wave issues its
-// share (2 + 2 instructions) of K(j+2) and V(j+1) from inside its MFMA phase j,
-// where the address arithmetic and the issue ride under the matrix pipe, and
-// waits for them (vmcnt) at the end of its MFMA phase j+1; both tiles are first
-// read in MFMA phase j+2 / j+1's successor, at least three slots after issue.
-// The buffers they overwrite held K(j-1) and V(j-2), last read in MFMA phase
-// j-1 of either group, which ended at least one barrier before any wave's
-// phase j began. Past the last tile the loads re-fetch the last tile into a
-// buffer nobody reads, which keeps the issue and wait counts constant.
 constexpr int kPpBM = 256;
 constexpr int kStages = 3;
 constexpr int kPpLdsBytes = 2 * kStages * kTileBytes;   // K[3], V[3] = 96 KB
@@ -516,34 +257,19 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
 
 // ---- host launchers -------------------------------------------------------------
 
-extern "C" int fv_internal_flash_block_m(void) {
-    static const int bm = [] {
-        const char* e = getenv("FV_FLASH_KERNEL");
-        return (e && e[0] == 'v' && e[1] == '1') ? fv::kBM : fv::kPpBM;
-    }();
-    return bm;
-}
+extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 
 extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal,
                                                hipStream_t stream) {
-    const bool pp = fv_internal_flash_block_m() == fv::kPpBM;
-    static bool attr_done[4] = {false, false, false, false};
-    const void* fn = pp ? (causal ? (const void*)fv::flash_fwd_pp_d128<true> : (const void*)fv::flash_fwd_pp_d128<false>)
-                        : (causal ? (const void*)fv::flash_fwd_d128<true> : (const void*)fv::flash_fwd_d128<false>);
-    const int lds = pp ? fv::kPpLdsBytes : fv::kFlashLdsBytes;
-    const int idx = (pp ? 2 : 0) + causal;
-    if (!attr_done[idx]) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    static bool attr_done[2] = {false, false};
+    const void* fn = causal ? (const void*)fv::flash_fwd_pp_d128<true> : (const void*)fv::flash_fwd_pp_d128<false>;
+    if (!attr_done[causal ? 1 : 0]) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, fv::kPpLdsBytes);
         if (e != hipSuccess) return e;
-        attr_done[idx] = true;
+        attr_done[causal ? 1 : 0] = true;
     }
-    const dim3 grid(p->per_xcd * 8), block(pp ? 512 : 256);
-    if (pp) {
-        if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp_d128<true>, grid, block, lds, stream, *p);
-        else hipLaunchKernelGGL(fv::flash_fwd_pp_d128<false>, grid, block, lds, stream, *p);
-    } else {
-        if (causal) hipLaunchKernelGGL(fv::flash_fwd_d128<true>, grid, block, lds, stream, *p);
-        else hipLaunchKernelGGL(fv::flash_fwd_d128<false>, grid, block, lds, stream, *p);
-    }
+    const dim3 grid(p->per_xcd * 8), block(512);
+    if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp_d128<true>, grid, block, fv::kPpLdsBytes, stream, *p);
+    else hipLaunchKernelGGL(fv::flash_fwd_pp_d128<false>, grid, block, fv::kPpLdsBytes, stream, *p);
     return hipGetLastError();
 }

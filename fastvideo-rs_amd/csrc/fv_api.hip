@@ -11,11 +11,6 @@
 #include "fv_internal.h"
 
 static thread_local std::string g_last_error;
-#ifdef FV_PROF
-void* g_fv_prof_buf = nullptr;
-extern "C" void* fv_prof_buf(void) { return g_fv_prof_buf; }
-#endif
-
 int fv_fail_hip(hipError_t e, const char* what) {
     char buf[256];
     snprintf(buf, sizeof buf, "%s: %s (hipError %d)", what, hipGetErrorString(e), (int)e);
@@ -67,14 +62,6 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
     p.k = k;
     p.v = v;
     p.out_f32 = out_is_bf16 ? nullptr : (float*)out;
-#ifdef FV_PROF
-    {
-        static void* dbg = nullptr;
-        if (!dbg) { (void)hipMalloc(&dbg, 8 * 512 * 8); (void)hipMemset(dbg, 0, 8 * 512 * 8); }
-        p.out_f32 = (float*)dbg;
-        ::g_fv_prof_buf = dbg;
-    }
-#endif
     p.out_bf16 = out_is_bf16 ? (uint16_t*)out : nullptr;
     p.out_is_bf16 = out_is_bf16 ? 1 : 0;
     p.sq = (int)sq;
