@@ -113,6 +113,35 @@ struct TileDma {
     static FV_DEV void issue_prepared(const Prepared& d, int it) {
         lds_dma16_s(d.lds + it * 4 * kRowBytes, (const void*)d.base, d.off[it]);
     }
+    // The same without per-descriptor lane offsets (scalars only): the tail clamp, needed by
+    // the last key tile alone, is then taken at issue time behind a wave-uniform branch.
+    struct Target {
+        unsigned long long base;
+        unsigned lds;
+        int rows_valid;
+    };
+    FV_DEV Target target(lds_u8* buf, const uint16_t* tile_base, int rows_valid, int wave) const {
+        Target d;
+        d.base = (unsigned long long)tile_base;
+        d.lds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 4 * kRowBytes);
+        d.rows_valid = rows_valid;
+        return d;
+    }
+    template <bool IS_V>
+    FV_DEV void issue_target(const Target& d) const {
+        if (d.rows_valid >= kTileRows) {
+#pragma unroll
+            for (int it = 0; it < ITER; it++)
+                lds_dma16_s(d.lds + it * 4 * kRowBytes, (const void*)d.base, IS_V ? voff[it] : koff[it]);
+        } else {
+#pragma unroll
+            for (int it = 0; it < ITER; it++) {
+                const unsigned off = IS_V ? voff[it] : koff[it];
+                const int over = max(0, (int)(off >> 8) - (d.rows_valid - 1));
+                lds_dma16_s(d.lds + it * 4 * kRowBytes, (const void*)d.base, off - over * kRowBytes);
+            }
+        }
+    }
     // tile_base (wave-uniform) points at the tile's first row. Rows >= rows_valid
     // re-read the last valid row: the caller masks their scores to -inf, so their
     // content only has to be finite data the tensor already holds.
@@ -240,6 +269,56 @@ FV_DEV void softmax_tile(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float
 #pragma unroll
             for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
             pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
+        }
+    }
+}
+
+// softmax_tile over a pair of tiles (128 keys) with one shared max / rescale decision.
+FV_DEV void softmax_tile_pair(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxState& st, f32x16 (&o)[4],
+                              float sl2, bf16x8 (&pb0)[4], bf16x8 (&pb1)[4]) {
+    const float NEG = neg_inf();
+    float mx = s0[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s0[0][i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s0[1][i]);
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s1[b][i]);
+    mx = pair_max(mx);
+    st.m_run = __builtin_fmaxf(st.m_run, mx);
+    const bool need = (st.m_run * sl2 - st.ms_used > kRescaleLog2) ||
+                      (st.m_used == NEG && st.m_run != NEG);
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {
+        const float ms_new = (st.m_run == NEG) ? 0.f : st.m_run * sl2;
+        const float alpha = (st.m_used == NEG) ? 0.f : fast_exp2(st.ms_used - ms_new);
+        st.l_acc *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
+        st.m_used = st.m_run;
+        st.ms_used = ms_new;
+    }
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            f32x16 e;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                e[i] = fast_exp2(__builtin_fmaf(half ? s1[b][i] : s0[b][i], sl2, -st.ms_used));
+                st.l_acc += e[i];
+            }
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                f32x8 f;
+#pragma unroll
+                for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
+                if (half) pb1[2 * b + t] = __builtin_convertvector(f, bf16x8);
+                else pb0[2 * b + t] = __builtin_convertvector(f, bf16x8);
+            }
         }
     }
 }

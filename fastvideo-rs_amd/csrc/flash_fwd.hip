@@ -253,6 +253,187 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
     }
 }
 
+// ---- dense variant: two key tiles per phase ----------------------------------------
+// The same two-group schedule with 128 keys per phase: a matrix phase is 64 MFMAs
+// (PV of the previous pair of tiles, QK of the current pair), a VALU phase two tile
+// softmaxes. Barriers, the LDS-latency ramp at the head of a matrix phase and the
+// per-phase bookkeeping are paid once per 128 keys. K and V tiles rotate through 4 LDS
+// buffers each (128 KB): matrix phase m reads K(2m), K(2m+1), V(2m-2), V(2m-1) and
+// issues K(2m+2), K(2m+3), V(2m), V(2m+1) into the buffers phase m-1 read last; every
+// wave waits for its own loads at the end of the same phase, one barrier before
+// phase m+1 of either group reads them. V buffers 2 and 3 start as zeros (phase 0
+// multiplies them with P = 0). An odd tile count is rounded up: the extra tile
+// re-reads the last one and all its scores are masked.
+constexpr int kRing2 = 4;
+constexpr int kPp2LdsBytes = 2 * kRing2 * kTileBytes;   // K[4], V[4] = 128 KB
+
+__global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    lds_u8* smem = (lds_u8*)smem_raw;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: branches on it stay scalar
+    const int grp = wave >> 2;
+    const int h = lane >> 5, c32 = lane & 31;
+    const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+    if (work >= p.total) return;
+    const int bh = work / p.nqt;
+    const int qt = work % p.nqt;
+    const int q0 = qt * kPpBM;
+    const int sq = p.sq, sk = p.sk;
+    const int qlen = min(kPpBM, sq - q0);
+    const float sl2 = p.sl2;
+    const float NEG = neg_inf();
+    // (see flash_fwd_pp_d128: scalar loads left pending at the loop head would turn every
+    // LDS wait count in the loop into a full drain)
+    float* out_f32 = p.out_f32;
+    uint16_t* out_bf16 = p.out_bf16;
+    int out_is_bf16 = p.out_is_bf16;
+    asm volatile("" : "+s"(out_f32), "+s"(out_bf16), "+s"(out_is_bf16));
+
+    const uint16_t* Qh = p.q + ((size_t)bh * sq + q0) * kD;
+    const uint16_t* Kh = p.k + (size_t)bh * sk * kD;
+    const uint16_t* Vh = p.v + (size_t)bh * sk * kD;
+
+    const int ne = (sk + kBN - 1) / kBN;     // key tiles
+    const int np = (ne + 1) / 2;             // phases
+    // tile t lives in buffer t mod 4 (t >= -2)
+    auto kbuf = [&](int t) -> lds_u8* { return smem + (t & (kRing2 - 1)) * kTileBytes; };
+    auto vbuf = [&](int t) -> lds_u8* { return smem + (kRing2 + (t & (kRing2 - 1))) * kTileBytes; };
+
+    TileDma<8> dma;
+    dma.init(wave, lane);
+    // tiles past the end repeat the last one
+    auto target_k = [&](int t) {
+        const int kv0 = min(t, ne - 1) * kBN;
+        return dma.prepare<false>(kbuf(t), Kh + (size_t)kv0 * kD, sk - kv0, wave);
+    };
+    auto target_v = [&](int t) {
+        const int kv0 = min(t, ne - 1) * kBN;
+        return dma.prepare<true>(vbuf(t), Vh + (size_t)kv0 * kD, sk - kv0, wave);
+    };
+    {
+        const TileDma<8>::Prepared a0 = target_k(0), a1 = target_k(1);
+        TileDma<8>::issue_prepared(a0, 0);
+        TileDma<8>::issue_prepared(a0, 1);
+        TileDma<8>::issue_prepared(a1, 0);
+        TileDma<8>::issue_prepared(a1, 1);
+    }
+    {   // zero V buffers 2 and 3: 32 KB, 64 B per thread
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        lds_u8* zb = smem + (kRing2 + 2) * kTileBytes + tid * 64;
+#pragma unroll
+        for (int i = 0; i < 4; i++) lds_write_b128(zb + 16 * i, z);
+    }
+    bf16x8 qf[8];
+    {
+        const int row = wave * 32 + c32;
+        load_q_frags(Qh, row, row < qlen, lane, qf);   // drains vmcnt: K(0), K(1) have landed too
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the zero fill is in LDS
+    const TileReadBases rb = tile_read_bases(lane);
+
+    f32x16 o[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[db][i] = 0.f;
+    SoftmaxState st;
+    st.init();
+    f32x16 s0[2], s1[2];
+    bf16x8 pb0[4], pb1[4];     // P of the previous pair of tiles; zero before the first
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int x = 0; x < 8; x++) {
+            pb0[t][x] = (__bf16)0.0f;
+            pb1[t][x] = (__bf16)0.0f;
+        }
+
+    TileDma<8>::Prepared dk0 = target_k(2), dk1 = target_k(3), dv0 = target_v(0), dv1 = target_v(1);
+
+    block_barrier();                 // K(0), K(1), zeros resident
+    if (grp == 1) block_barrier();   // group 1 idles through slot 0
+
+    auto mask_tail = [&](f32x16 (&s)[2], int kv0) {
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
+                if (key >= sk) s[b][i] = NEG;
+            }
+    };
+
+#pragma unroll 1
+    for (int m = 0; m < np; m++) {
+        // ---- matrix phase: group 0 in slot 2m, group 1 in slot 2m+1 ----
+        __builtin_amdgcn_s_setprio(1);
+        constexpr int kAhead = 3;
+        mfma_phase<true, kAhead>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, [&](int g) {
+            if (g == 1) TileDma<8>::issue_prepared(dk0, 0);
+            if (g == 2) TileDma<8>::issue_prepared(dk0, 1);
+            if (g == 4) TileDma<8>::issue_prepared(dk1, 0);
+            if (g == 5) TileDma<8>::issue_prepared(dk1, 1);
+        });
+        mfma_phase<true, kAhead>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, [&](int g) {
+            if (g == 1) TileDma<8>::issue_prepared(dv0, 0);
+            if (g == 2) TileDma<8>::issue_prepared(dv0, 1);
+            if (g == 4) TileDma<8>::issue_prepared(dv1, 0);
+            if (g == 5) TileDma<8>::issue_prepared(dv1, 1);
+        });
+        __builtin_amdgcn_s_setprio(0);
+        wait_vmcnt<0>();             // this wave's loads of this phase have landed
+        __builtin_amdgcn_sched_barrier(0);
+        block_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- VALU phase: group 0 in slot 2m+1, group 1 in slot 2m+2 ----
+        if (2 * (m + 1) * kBN > sk) {
+            mask_tail(s0, 2 * m * kBN);
+            mask_tail(s1, (2 * m + 1) * kBN);
+        }
+        softmax_tile_pair(s0, s1, st, o, sl2, pb0, pb1);
+        // P and the row sum must be complete before the barrier: without this the
+        // compiler sinks the exponentials past it, into the matrix phase
+        asm volatile("" ::"v"(pb0[0]), "v"(pb0[1]), "v"(pb0[2]), "v"(pb0[3]), "v"(pb1[0]), "v"(pb1[1]),
+                     "v"(pb1[2]), "v"(pb1[3]), "v"(st.l_acc));
+        dk0 = target_k(2 * m + 4);   // for matrix phase m+1
+        dk1 = target_k(2 * m + 5);
+        dv0 = target_v(2 * m + 2);
+        dv1 = target_v(2 * m + 3);
+        if (grp == 0 || m + 1 < np) {
+            __builtin_amdgcn_sched_barrier(0);
+            block_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // O += P V of the last pair (their V landed before the last barrier both groups passed)
+    pv_tile(vbuf(2 * np - 2), rb.v, pb0, o);
+    pv_tile(vbuf(2 * np - 1), rb.v, pb1, o);
+
+    const float l_tot = pair_sum(st.l_acc);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int row = wave * 32 + c32;
+    if (row < qlen) {
+        const size_t base = ((size_t)bh * sq + q0 + row) * kD;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d0 = 32 * db + 8 * g + 4 * h;
+                f32x4 r;
+#pragma unroll
+                for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
+                if (out_is_bf16) {
+                    const bf16x4 rb4 = __builtin_convertvector(r, bf16x4);
+                    *reinterpret_cast<bf16x4*>(out_bf16 + base + d0) = rb4;
+                } else {
+                    *reinterpret_cast<f32x4*>(out_f32 + base + d0) = r;
+                }
+            }
+    }
+}
+
 }  // namespace fv
 
 // ---- host launchers -------------------------------------------------------------
@@ -262,14 +443,15 @@ extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal,
                                                hipStream_t stream) {
     static bool attr_done[2] = {false, false};
-    const void* fn = causal ? (const void*)fv::flash_fwd_pp_d128<true> : (const void*)fv::flash_fwd_pp_d128<false>;
+    const void* fn = causal ? (const void*)fv::flash_fwd_pp_d128<true> : (const void*)fv::flash_fwd_pp2_d128;
+    const int lds = causal ? fv::kPpLdsBytes : fv::kPp2LdsBytes;
     if (!attr_done[causal ? 1 : 0]) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, fv::kPpLdsBytes);
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
         attr_done[causal ? 1 : 0] = true;
     }
     const dim3 grid(p->per_xcd * 8), block(512);
-    if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp_d128<true>, grid, block, fv::kPpLdsBytes, stream, *p);
-    else hipLaunchKernelGGL(fv::flash_fwd_pp_d128<false>, grid, block, fv::kPpLdsBytes, stream, *p);
+    if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp_d128<true>, grid, block, lds, stream, *p);
+    else hipLaunchKernelGGL(fv::flash_fwd_pp2_d128, grid, block, lds, stream, *p);
     return hipGetLastError();
 }

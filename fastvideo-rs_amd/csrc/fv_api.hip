@@ -82,9 +82,13 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
         p.ft = (int)block_tokens;
         p.win = (int)window;
         p.sink = (int)sink;
+        // One block spanning both sequences: every key is visible to every query (tq == tk == 0
+        // for any window), so this is the dense problem and runs on the dense kernel, bit for bit
+        // (the reference asserts that identity for its own kernels, gpucheck kernels_wan.rs:230-261).
+        if (block_tokens >= sq && block_tokens >= sk) causal = false;
     }
     hipError_t e = fv_internal_launch_flash(&p, causal ? 1 : 0, (hipStream_t)stream);
-    if (e != hipSuccess) return fail_hip(e, causal ? "flash_fwd_d128<causal>" : "flash_fwd_d128");
+    if (e != hipSuccess) return fail_hip(e, causal ? "flash_fwd_pp_d128<causal>" : "flash_fwd_pp2_d128");
     return FV_OK;
 }
 
