@@ -261,7 +261,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.out_bf16 else None,
-                     "kernel": "fv::flash_fwd_pp_d128<true>" if bt else "fv::flash_fwd_pp2_d128",
+                     "kernel": "fv::flash_fwd_pp2_d128<true>" if bt else "fv::flash_fwd_pp2_d128<false>",
                      "avg_kernel_ms": round(avg_kernel_ms, 4), "median_kernel_ms": round(kern_ms[len(kern_ms) // 2], 4),
                      "min_hbm_bytes": bytes_min,
                      "hbm_frac_at_min_traffic": round(bytes_min / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},

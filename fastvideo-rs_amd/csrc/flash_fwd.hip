@@ -30,21 +30,29 @@
 //     loses on this hardware: a wave issues in order, so its VALU work stalls
 //     behind every MFMA that waits for the matrix pipe;
 //   * K/V tiles go global -> LDS directly (global_load_lds_dwordx4) into
-//     XOR-swizzled unpadded tiles, three stages each;
+//     XOR-swizzled unpadded tiles, four buffers each;
 //   * workgroup ids are remapped so that the workgroups resident on one XCD
 //     walk consecutive query tiles of the same head (their K/V stream hits
 //     that XCD's L2).
 //
-// Time is counted in slots (one phase each). Group 0 runs MFMA(j) in slot 2j and
-// VALU(j) in slot 2j+1; group 1 is one slot behind. Every wave issues its
-// share (2 + 2 instructions) of K(j+2) and V(j+1) from inside its MFMA phase j,
-// from descriptors (addresses, tail clamp) prepared in the VALU phase before,
-// and waits for them (vmcnt) at the end of its MFMA phase j+1; both tiles are
-// first read at least three slots after issue. The buffers they overwrite held
-// K(j-1) and V(j-2), last read in MFMA phase j-1 of either group, which ended
-// at least one barrier before any wave's phase j began. Past the last tile the
-// loads re-fetch the last tile into a buffer nobody reads, which keeps the
-// issue and wait counts constant.
+// Time is counted in slots (one phase each); a phase covers a PAIR of key tiles
+// (128 keys): a matrix phase is 64 MFMAs (PV of the previous pair, QK of the
+// current pair), a VALU phase the softmax of the pair with one shared max /
+// rescale decision. Barriers, the LDS-latency ramp at the head of a matrix phase
+// and the per-phase bookkeeping are thus paid once per 128 keys. Group 0 runs
+// matrix phase m in slot 2m and VALU phase m in slot 2m+1; group 1 is one slot
+// behind. K and V tiles rotate through 4 LDS buffers each (128 KB): matrix phase
+// m reads K(2m), K(2m+1), V(2m-2), V(2m-1) and issues K(2m+2), K(2m+3), V(2m),
+// V(2m+1) into the buffers phase m-1 read last, from descriptors (addresses, tail
+// clamp) prepared in the VALU phase before, so the matrix phase carries bare DMA
+// instructions and no branches (a branch inside the unrolled phase breaks the
+// register allocation of the 16-register accumulator tuples: 59 spills measured).
+// Every wave waits for its own loads at the end of the same phase, one barrier
+// before phase m+1 of either group reads them. V buffers 2 and 3 start as zeros
+// (phase 0 multiplies them with P = 0). An odd tile count is rounded up: the extra
+// tile re-reads the last one and all its scores are masked. Tile indices are walk
+// positions: for block-causal calls the walk is the sink tiles [0, ns) followed
+// by the band [mlo, mhi).
 #include "attn_core.h"
 #include "fv_internal.h"
 
@@ -53,12 +61,13 @@ namespace fv {
 constexpr int kD = 128;          // head dim
 constexpr int kBN = 64;          // keys per tile
 
-constexpr int kPpBM = 256;
-constexpr int kStages = 3;
-constexpr int kPpLdsBytes = 2 * kStages * kTileBytes;   // K[3], V[3] = 96 KB
+constexpr int kPpBM = 256;      // queries per workgroup
+
+constexpr int kRing2 = 4;
+constexpr int kPp2LdsBytes = 2 * kRing2 * kTileBytes;   // K[4], V[4] = 128 KB
 
 template <bool CAUSAL>
-__global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p) {
+__global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     lds_u8* smem = (lds_u8*)smem_raw;
 
@@ -88,7 +97,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
     const uint16_t* Vh = p.v + (size_t)bh * sk * kD;
 
     const int nkt = (sk + kBN - 1) / kBN;
-    int ns = 0, mlo = 0, ne = nkt;
+    int ns = 0, mlo = 0, ne = nkt;           // walk: tiles [0, ns) then [mlo, mlo + ne - ns)
     int hi_q = 0, lo_q = 0, sink_tok = 0;
     if constexpr (CAUSAL) {
         const int ft = p.ft, win = p.win;
@@ -106,197 +115,13 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp_d128(const FlashParams p)
         lo_q = win > 0 ? max(0, tq - win + 1) * ft : 0;
     }
     if (ne <= 0) return;   // cannot happen for sk >= 1 (the walk always holds the query's own block)
-    // key-tile index of walk position e; positions past the end repeat the last tile
-    auto tile_of = [&](int e) -> int {
-        e = min(e, ne - 1);
-        if constexpr (CAUSAL) return e < ns ? e : mlo + (e - ns);
-        else return e;
-    };
-    auto kbuf = [&](int st) -> lds_u8* { return smem + st * kTileBytes; };
-    auto vbuf = [&](int st) -> lds_u8* { return smem + (kStages + st) * kTileBytes; };
-    auto next_stage = [](int st) -> int { return st == kStages - 1 ? 0 : st + 1; };
-
-    TileDma<8> dma;
-    dma.init(wave, lane);
-    auto issue_k = [&](int e, int st) {
-        const int kv0 = tile_of(e) * kBN;
-        dma.issue<false>(kbuf(st), Kh + (size_t)kv0 * kD, sk - kv0, wave);
-    };
-    auto issue_v = [&](int e, int st) {
-        const int kv0 = tile_of(e) * kBN;
-        dma.issue<true>(vbuf(st), Vh + (size_t)kv0 * kD, sk - kv0, wave);
-    };
-
-    issue_k(0, 0);
-    issue_k(1, 1);
-    issue_v(0, 0);
-    bf16x8 qf[8];
-    {
-        const int row = wave * 32 + c32;
-        load_q_frags(Qh, row, row < qlen, lane, qf);   // drains vmcnt: the three tiles have landed too
-    }
-    const TileReadBases rb = tile_read_bases(lane);
-
-    f32x16 o[4];
-#pragma unroll
-    for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) o[db][i] = 0.f;
-    SoftmaxState st;
-    st.init();
-    f32x16 s[2];
-    bf16x8 pb[4];     // P of the previous tile; zero before the first one
-#pragma unroll
-    for (int t = 0; t < 4; t++)
-#pragma unroll
-        for (int x = 0; x < 8; x++) pb[t][x] = (__bf16)0.0f;
-
-    // the loads a matrix phase issues are prepared (addresses, tail clamp) one VALU phase earlier
-    auto prep_k = [&](int e, int st) {
-        const int kv0 = tile_of(e) * kBN;
-        return dma.prepare<false>(kbuf(st), Kh + (size_t)kv0 * kD, sk - kv0, wave);
-    };
-    auto prep_v = [&](int e, int st) {
-        const int kv0 = tile_of(e) * kBN;
-        return dma.prepare<true>(vbuf(st), Vh + (size_t)kv0 * kD, sk - kv0, wave);
-    };
-    TileDma<8>::Prepared dk = prep_k(2, 2), dv = prep_v(1, 1);
-
-    block_barrier();                 // K(0), K(1), V(0) resident
-    if (grp == 1) block_barrier();   // group 1 idles through slot 0
-
-    // LDS stages: K(j) in sk_cur, K(j+2) goes to sk_ld = stage of j-1; V(j-1) in sv_prev, V(j+1)
-    // goes to the stage after V(j)
-    int sk_cur = 0, sk_ld = 2, sv_prev = 0, sv_ld = 1;
-#pragma unroll 1
-    for (int j = 0; j < ne; j++) {
-        // ---- MFMA phase: group 0 in slot 2j, group 1 in slot 2j+1 ----
-        __builtin_amdgcn_s_setprio(1);
-        constexpr int kAhead = CAUSAL ? 2 : 3;   // LDS prefetch depth the register budget allows
-        // P starts as zero, so the first pass adds 0 * V(0) (finite, resident) and needs no special case
-        mfma_phase<true, kAhead>(vbuf(sv_prev), kbuf(sk_cur), rb, pb, o, qf, s, [&](int g) {
-            if (g == 1) TileDma<8>::issue_prepared(dk, 0);
-            if (g == 2) TileDma<8>::issue_prepared(dk, 1);
-            if (g == 4) TileDma<8>::issue_prepared(dv, 0);
-            if (g == 5) TileDma<8>::issue_prepared(dv, 1);
-        });
-        __builtin_amdgcn_s_setprio(0);
-        wait_vmcnt<4>();             // this wave's loads of the previous phase have landed
-        __builtin_amdgcn_sched_barrier(0);
-        block_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- VALU phase: group 0 in slot 2j+1, group 1 in slot 2j+2 ----
-        const int kv0 = tile_of(j) * kBN;
-        if (kv0 + kBN > sk) {
-#pragma unroll
-            for (int b = 0; b < 2; b++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
-                    if (key >= sk) s[b][i] = NEG;
-                }
-        }
-        if constexpr (CAUSAL) {
-            const int kend = min(kv0 + kBN, sk);
-            const bool lane_all = (kend <= hi_q && kv0 >= lo_q) || kend <= sink_tok;
-            if (__builtin_amdgcn_ballot_w64(!lane_all) != 0) {
-#pragma unroll
-                for (int b = 0; b < 2; b++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
-                        const bool vis = (key < hi_q && key >= lo_q) || key < sink_tok;
-                        if (!vis) s[b][i] = NEG;
-                    }
-            }
-        }
-        softmax_tile(s, st, o, sl2, pb);
-        // P and the row sum must be complete before the barrier: without this the
-        // compiler sinks the exponentials past it, into the matrix phase
-        asm volatile("" ::"v"(pb[0]), "v"(pb[1]), "v"(pb[2]), "v"(pb[3]), "v"(st.l_acc));
-        sv_prev = j > 0 ? next_stage(sv_prev) : 0;   // V(j) lives in stage j % 3
-        sv_ld = next_stage(sv_ld);
-        sk_ld = sk_cur;
-        sk_cur = next_stage(sk_cur);
-        dk = prep_k(j + 3, sk_ld);   // for matrix phase j+1: K(j+3), V(j+2)
-        dv = prep_v(j + 2, sv_ld);
-        if (grp == 0 || j + 1 < ne) {
-            __builtin_amdgcn_sched_barrier(0);
-            block_barrier();
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    // O += P V of the last tile (its V landed before the last barrier both groups passed)
-    pv_tile(vbuf(sv_prev), rb.v, pb, o);
-    wait_vmcnt<0>();   // the redundant tail loads must not outlive the workgroup's LDS
-
-    const float l_tot = pair_sum(st.l_acc);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    const int row = wave * 32 + c32;
-    if (row < qlen) {
-        const size_t base = ((size_t)bh * sq + q0 + row) * kD;
-#pragma unroll
-        for (int db = 0; db < 4; db++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int d0 = 32 * db + 8 * g + 4 * h;
-                f32x4 r;
-#pragma unroll
-                for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
-                if (out_is_bf16) {
-                    const bf16x4 rb4 = __builtin_convertvector(r, bf16x4);
-                    *reinterpret_cast<bf16x4*>(out_bf16 + base + d0) = rb4;
-                } else {
-                    *reinterpret_cast<f32x4*>(out_f32 + base + d0) = r;
-                }
-            }
-    }
-}
-
-// ---- dense variant: two key tiles per phase ----------------------------------------
-// The same two-group schedule with 128 keys per phase: a matrix phase is 64 MFMAs
-// (PV of the previous pair of tiles, QK of the current pair), a VALU phase two tile
-// softmaxes. Barriers, the LDS-latency ramp at the head of a matrix phase and the
-// per-phase bookkeeping are paid once per 128 keys. K and V tiles rotate through 4 LDS
-// buffers each (128 KB): matrix phase m reads K(2m), K(2m+1), V(2m-2), V(2m-1) and
-// issues K(2m+2), K(2m+3), V(2m), V(2m+1) into the buffers phase m-1 read last; every
-// wave waits for its own loads at the end of the same phase, one barrier before
-// phase m+1 of either group reads them. V buffers 2 and 3 start as zeros (phase 0
-// multiplies them with P = 0). An odd tile count is rounded up: the extra tile
-// re-reads the last one and all its scores are masked.
-constexpr int kRing2 = 4;
-constexpr int kPp2LdsBytes = 2 * kRing2 * kTileBytes;   // K[4], V[4] = 128 KB
-
-__global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    lds_u8* smem = (lds_u8*)smem_raw;
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: branches on it stay scalar
-    const int grp = wave >> 2;
-    const int h = lane >> 5, c32 = lane & 31;
-    const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-    if (work >= p.total) return;
-    const int bh = work / p.nqt;
-    const int qt = work % p.nqt;
-    const int q0 = qt * kPpBM;
-    const int sq = p.sq, sk = p.sk;
-    const int qlen = min(kPpBM, sq - q0);
-    const float sl2 = p.sl2;
-    const float NEG = neg_inf();
-    // (see flash_fwd_pp_d128: scalar loads left pending at the loop head would turn every
-    // LDS wait count in the loop into a full drain)
-    float* out_f32 = p.out_f32;
-    uint16_t* out_bf16 = p.out_bf16;
-    int out_is_bf16 = p.out_is_bf16;
-    asm volatile("" : "+s"(out_f32), "+s"(out_bf16), "+s"(out_is_bf16));
-
-    const uint16_t* Qh = p.q + ((size_t)bh * sq + q0) * kD;
-    const uint16_t* Kh = p.k + (size_t)bh * sk * kD;
-    const uint16_t* Vh = p.v + (size_t)bh * sk * kD;
-
-    const int ne = (sk + kBN - 1) / kBN;     // key tiles
     const int np = (ne + 1) / 2;             // phases
+    // first key of walk position e; positions past the end repeat the last tile (their scores are masked)
+    auto kv0_of = [&](int e) -> int {
+        e = min(e, ne - 1);
+        if constexpr (CAUSAL) return (e < ns ? e : mlo + (e - ns)) * kBN;
+        else return e * kBN;
+    };
     // tile t lives in buffer t mod 4 (t >= -2)
     auto kbuf = [&](int t) -> lds_u8* { return smem + (t & (kRing2 - 1)) * kTileBytes; };
     auto vbuf = [&](int t) -> lds_u8* { return smem + (kRing2 + (t & (kRing2 - 1))) * kTileBytes; };
@@ -305,11 +130,11 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
     dma.init(wave, lane);
     // tiles past the end repeat the last one
     auto target_k = [&](int t) {
-        const int kv0 = min(t, ne - 1) * kBN;
+        const int kv0 = kv0_of(t);
         return dma.prepare<false>(kbuf(t), Kh + (size_t)kv0 * kD, sk - kv0, wave);
     };
     auto target_v = [&](int t) {
-        const int kv0 = min(t, ne - 1) * kBN;
+        const int kv0 = kv0_of(t);
         return dma.prepare<true>(vbuf(t), Vh + (size_t)kv0 * kD, sk - kv0, wave);
     };
     {
@@ -355,21 +180,42 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
     block_barrier();                 // K(0), K(1), zeros resident
     if (grp == 1) block_barrier();   // group 1 idles through slot 0
 
-    auto mask_tail = [&](f32x16 (&s)[2], int kv0) {
+    // scores of walk position e: keys past the end (or a position past the walk) to -inf;
+    // block-causal: keys this lane's query may not see to -inf, skipped when the whole
+    // wave sees the whole tile
+    auto mask_tile = [&](f32x16 (&s)[2], int e) {
+        const int kv0 = kv0_of(e);
+        if (e >= ne || kv0 + kBN > sk) {
+            const int lim = e >= ne ? 0 : sk;
 #pragma unroll
-        for (int b = 0; b < 2; b++)
+            for (int b = 0; b < 2; b++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
-                if (key >= sk) s[b][i] = NEG;
+                for (int i = 0; i < 16; i++) {
+                    const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
+                    if (key >= lim) s[b][i] = NEG;
+                }
+        }
+        if constexpr (CAUSAL) {
+            const int kend = min(kv0 + kBN, sk);
+            const bool lane_all = (kend <= hi_q && kv0 >= lo_q) || kend <= sink_tok;
+            if (__builtin_amdgcn_ballot_w64(!lane_all) != 0) {
+#pragma unroll
+                for (int b = 0; b < 2; b++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
+                        const bool vis = (key < hi_q && key >= lo_q) || key < sink_tok;
+                        if (!vis) s[b][i] = NEG;
+                    }
             }
+        }
     };
 
 #pragma unroll 1
     for (int m = 0; m < np; m++) {
         // ---- matrix phase: group 0 in slot 2m, group 1 in slot 2m+1 ----
         __builtin_amdgcn_s_setprio(1);
-        constexpr int kAhead = 3;
+        constexpr int kAhead = CAUSAL ? 2 : 3;
         mfma_phase<true, kAhead>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, [&](int g) {
             if (g == 1) TileDma<8>::issue_prepared(dk0, 0);
             if (g == 2) TileDma<8>::issue_prepared(dk0, 1);
@@ -388,10 +234,8 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
         block_barrier();
         __builtin_amdgcn_sched_barrier(0);
         // ---- VALU phase: group 0 in slot 2m+1, group 1 in slot 2m+2 ----
-        if (2 * (m + 1) * kBN > sk) {
-            mask_tail(s0, 2 * m * kBN);
-            mask_tail(s1, (2 * m + 1) * kBN);
-        }
+        mask_tile(s0, 2 * m);
+        mask_tile(s1, 2 * m + 1);
         softmax_tile_pair(s0, s1, st, o, sl2, pb0, pb1);
         // P and the row sum must be complete before the barrier: without this the
         // compiler sinks the exponentials past it, into the matrix phase
@@ -443,15 +287,15 @@ extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal,
                                                hipStream_t stream) {
     static bool attr_done[2] = {false, false};
-    const void* fn = causal ? (const void*)fv::flash_fwd_pp_d128<true> : (const void*)fv::flash_fwd_pp2_d128;
-    const int lds = causal ? fv::kPpLdsBytes : fv::kPp2LdsBytes;
+    const void* fn = causal ? (const void*)fv::flash_fwd_pp2_d128<true> : (const void*)fv::flash_fwd_pp2_d128<false>;
+    const int lds = fv::kPp2LdsBytes;
     if (!attr_done[causal ? 1 : 0]) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
         attr_done[causal ? 1 : 0] = true;
     }
     const dim3 grid(p->per_xcd * 8), block(512);
-    if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp_d128<true>, grid, block, lds, stream, *p);
-    else hipLaunchKernelGGL(fv::flash_fwd_pp2_d128, grid, block, lds, stream, *p);
+    if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp2_d128<true>, grid, block, lds, stream, *p);
+    else hipLaunchKernelGGL(fv::flash_fwd_pp2_d128<false>, grid, block, lds, stream, *p);
     return hipGetLastError();
 }

@@ -88,7 +88,7 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
         if (block_tokens >= sq && block_tokens >= sk) causal = false;
     }
     hipError_t e = fv_internal_launch_flash(&p, causal ? 1 : 0, (hipStream_t)stream);
-    if (e != hipSuccess) return fail_hip(e, causal ? "flash_fwd_pp_d128<causal>" : "flash_fwd_pp2_d128");
+    if (e != hipSuccess) return fail_hip(e, causal ? "flash_fwd_pp2_d128<true>" : "flash_fwd_pp2_d128<false>");
     return FV_OK;
 }
 
