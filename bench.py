@@ -8,7 +8,7 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny|vsa624|vsa512) are for the
+Other workloads (--workload cross|causal|causal3|c5|tiny|vsa624|vsa512|prep) are for the
 design notes; the driver's line is the default `self`.
 """
 import argparse
@@ -115,6 +115,71 @@ def bench_vsa(args):
     print(json.dumps(rec), flush=True)
 
 
+def bench_prep(args):
+    """The producer / consumer either side of the SDPA call at the headline shape: q and k
+    RMSNorm + RoPE (bf16 kernel) and the V split out of a fused bf16 QKV projection
+    [1, 32760, 3*1536], and merge_heads of the attention output. HBM-bound scans: the
+    figure is algorithmic bytes (each operand once) over HIP-event time."""
+    import torch
+
+    import fv_sdpa
+
+    fv_sdpa.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    batch, seq, heads, d = 1, 32760, 12, 128
+    width = heads * d
+    g = torch.Generator(device=dev).manual_seed(20242)
+    proj = torch.randn((batch, seq, 3 * width), generator=g, device=dev).to(torch.bfloat16)
+    w = (1.0 + 0.1 * torch.randn(width, generator=g, device=dev)).float()
+    ang = torch.rand((seq, d // 2), generator=g, device=dev) * 6.0 - 3.0
+    cos = torch.cos(ang).repeat_interleave(2, dim=1).contiguous()
+    sin = torch.sin(ang).repeat_interleave(2, dim=1).contiguous()
+    o = torch.randn((batch, heads, seq, d), generator=g, device=dev).to(torch.bfloat16)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        t0 = time.perf_counter()
+        for a, b in evs:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / args.steps
+        ms = sorted(a.elapsed_time(b) for a, b in evs)
+        return wall, sum(ms) / len(ms)
+
+    row = seq * width * 2
+    tables = 2 * seq * d * 4
+    ops = {
+        "qk_norm_rope_bhsd (bf16, rope)": (lambda: fv_sdpa.qk_norm_rope_bhsd(proj, 0, heads, w, (cos, sin)),
+                                           2 * row + tables + width * 4),
+        "split_heads_bhsd (bf16)": (lambda: fv_sdpa.split_heads_bhsd(proj, 2 * width, heads, d), 2 * row),
+        "merge_heads (bf16)": (lambda: fv_sdpa.merge_heads(o), 2 * row),
+    }
+    res = {}
+    for name, (fn, nbytes) in ops.items():
+        wall, avg = timed(fn)
+        res[name] = {"avg_kernel_ms": round(avg, 4), "ms_per_step": round(wall, 4), "algorithmic_bytes": nbytes,
+                     "GBps": round(nbytes / (avg * 1e-3) / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+    main_op = res["qk_norm_rope_bhsd (bf16, rope)"]
+    rec = {
+        "metric": "q/k RMSNorm+RoPE -> BHSD GB/s (Wan-1.3B 480p, bf16)", "value": main_op["GBps"], "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_op["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "fused QKV projection [1,32760,4608] bf16 -> q/k/v BHSD, H=12 d=128; merge of [1,12,32760,128]"},
+        "ops": res,
+        "roofline": {"bound": "hbm", "achieved": main_op["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": main_op["frac_of_hbm_peak"], "traffic": None, "kernel": "fv::qk_norm_rope_bhsd_kernel",
+                     "avg_kernel_ms": main_op["avg_kernel_ms"]},
+    }
+    print(json.dumps(rec), flush=True)
+
+
 def visible_pairs(sq, sk, bt):
     if bt == 0:
         return sq * sk
@@ -165,7 +230,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS))
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -186,6 +251,9 @@ def main():
         sys.exit(3)
     if args.workload in VSA_WORKLOADS:
         bench_vsa(args)
+        return
+    if args.workload == "prep":
+        bench_prep(args)
         return
     fv_sdpa.lib()
     dev = torch.device("cuda:0")

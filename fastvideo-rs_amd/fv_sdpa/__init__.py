@@ -6,3 +6,4 @@ from ._lib import FvDeclined, FvError, LIB_PATH, build, lib  # noqa: F401
 from .ops import *  # noqa: F401,F403
 from .vsa import *  # noqa: F401,F403
 from .sdpa import *  # noqa: F401,F403
+from .prep import *  # noqa: F401,F403

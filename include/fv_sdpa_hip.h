@@ -172,6 +172,29 @@ int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf1
                      void* workspace, size_t workspace_bytes, uint32_t* selected_out, size_t bh,
                      size_t seq, size_t num_tiles, size_t topk, size_t dim, float scale, void* stream);
 
+/* ---- producer / consumer either side of the SDPA call --------------------------------- */
+/* q/k RMSNorm across all heads (+ interleaved RoPE) of columns [col_off, col_off + heads*d) of
+ * src [batch, seq, src_width], written as BHSD [batch, heads, seq, d].
+ * out_is_bf16 == 0: the f32 op, `x*inv*w`, rotation, f32 out — rt/ops.rs:528-572 /
+ *   kernels/core.cu:373-413 `qk_norm_rope_bhsd` (host form rt/ops.rs:2304-2350).
+ * out_is_bf16 == 1: the bf16 q/k kernel with its rounding points, `bf16(bf16(x*inv)*w)`, rotation
+ *   in f32, one rounding, bf16 out — wan/fuse.rs:527-561 `wan_qk_norm_rope16` (policy
+ *   rt/fuse/policy.rs:404-412, host twin rt/fuse/host.rs:217-276).
+ * src and w are f32 or bf16 (flags); cos_t / sin_t are f32 [seq, d] (cos read from the even slot
+ * of a pair, sin from the odd one) or both NULL for no rotation. Declines unless d, col_off and
+ * src_width are multiples of 8. */
+int fv_qk_norm_rope_bhsd(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
+                         const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
+                         size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
+                         size_t col_off, float eps, void* stream);
+/* rt/ops.rs:574-602 / kernels/core.cu:415-427 `split_heads_bhsd`: the value heads, a pure permute
+ * of f32 or bf16 elements. */
+int fv_split_heads_bhsd(const void* src, void* out, int is_bf16, size_t batch, size_t seq, size_t heads,
+                        size_t d, size_t src_width, size_t col_off, void* stream);
+/* rt/ops.rs:604-620 / kernels/core.cu:429-443 `merge_heads`: BHSD -> [batch, seq, heads*d]. */
+int fv_merge_heads(const void* src, void* out, int is_bf16, size_t batch, size_t heads, size_t seq, size_t d,
+                   void* stream);
+
 /* ---- host-side mask / sharding helpers ------------------------------------------------ */
 /* rt/attn.rs:449-453 `BlockCausal::allows`. */
 int fv_block_causal_allows(size_t block_tokens, size_t window, size_t sink, size_t q, size_t k);

@@ -79,6 +79,10 @@ def _declare(l):
     l.fvo_vsa_tile_mean.argtypes = [_f32p, _i32p, _u32p, _f32p, _sz, _sz, _sz, _sz, C.c_int]
     l.fvo_vsa_coarse_scores.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, C.c_float]
     l.fvo_shard_ranges.argtypes = [_sz, _sz, _szp]
+    for fn in (l.fvo_qk_norm_rope_bhsd, l.fvo_wan_qk_norm_rope16):
+        fn.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _sz, _sz, _sz, _sz, _sz, _sz, C.c_float]
+    l.fvo_split_heads_bhsd.argtypes = [_f32p, _f32p, _sz, _sz, _sz, _sz, _sz, _sz]
+    l.fvo_merge_heads.argtypes = [_f32p, _f32p, _sz, _sz, _sz, _sz]
 
 
 def _f32(a):
@@ -318,3 +322,45 @@ def shard_ranges(seq, world):
     out = (C.c_size_t * (2 * w))()
     lib().fvo_shard_ranges(seq, world, out)
     return [(int(out[2 * r]), int(out[2 * r + 1])) for r in range(w)]
+
+
+# ---- producer / consumer either side of the SDPA call ---------------------------------
+
+def _qk(fn, proj, col_off, heads, w, rope, eps):
+    proj, w = _f32(proj), _f32(w)
+    batch, seq, src_width = proj.shape
+    d = w.size // heads
+    cos = sin = None
+    if rope is not None:
+        cos, sin = _f32(rope[0]), _f32(rope[1])
+        assert cos.shape == (seq, d) and sin.shape == (seq, d)
+    out = np.empty((batch, heads, seq, d), dtype=np.float32)
+    fn(_p(proj, _f32p), _p(w, _f32p), _p(cos, _f32p), _p(sin, _f32p), _p(out, _f32p), batch, seq, heads, d,
+       src_width, col_off, eps)
+    return out
+
+
+def qk_norm_rope_bhsd(proj, col_off, heads, w, rope=None, eps=1e-6):
+    """rt/ops.rs:2304-2350 (f32 op). proj [batch, seq, src_width], w [heads*d], rope (cos, sin) [seq, d]."""
+    return _qk(lib().fvo_qk_norm_rope_bhsd, proj, col_off, heads, w, rope, eps)
+
+
+def wan_qk_norm_rope16(proj, col_off, heads, w, rope=None, eps=1e-6):
+    """wan/fuse.rs:290-343 host twin (bf16 rounding points of WAN_QK_NORM_ROPE)."""
+    return _qk(lib().fvo_wan_qk_norm_rope16, proj, col_off, heads, w, rope, eps)
+
+
+def split_heads_bhsd(proj, col_off, heads, d):
+    proj = _f32(proj)
+    batch, seq, src_width = proj.shape
+    out = np.empty((batch, heads, seq, d), dtype=np.float32)
+    lib().fvo_split_heads_bhsd(_p(proj, _f32p), _p(out, _f32p), batch, seq, heads, d, src_width, col_off)
+    return out
+
+
+def merge_heads(x):
+    x = _f32(x)
+    batch, heads, seq, d = x.shape
+    out = np.empty((batch, seq, heads * d), dtype=np.float32)
+    lib().fvo_merge_heads(_p(x, _f32p), _p(out, _f32p), batch, heads, seq, d)
+    return out

@@ -550,3 +550,92 @@ void fvo_shard_ranges(size_t seq, size_t world, size_t* out) {
         start += len;
     }
 }
+
+/* ---- producer / consumer either side of the SDPA call --------------------------- */
+
+/* C/rt/ops.rs:2304-2350 */
+void fvo_qk_norm_rope_bhsd(const float* src, const float* w, const float* cos_t, const float* sin_t,
+                           float* out, size_t batch, size_t seq, size_t heads, size_t d,
+                           size_t src_width, size_t col_off, float eps) {
+    const size_t width = heads * d;
+    for (size_t b = 0; b < batch; b++)
+        for (size_t s = 0; s < seq; s++) {
+            const float* x = src + (b * seq + s) * src_width + col_off;
+            float ss = 0.0f;
+            for (size_t j = 0; j < width; j++) ss += x[j] * x[j];
+            const float ms = ss / (float)width;
+            const float inv = 1.0f / sqrtf(ms + eps);
+            for (size_t h = 0; h < heads; h++) {
+                float* o = out + ((b * heads + h) * seq + s) * d;
+                for (size_t p = 0; p < d; p++) {
+                    const size_t j = h * d + p;
+                    if (!cos_t || !sin_t) {
+                        o[p] = x[j] * inv * w[j];
+                    } else {
+                        const size_t even = p - (p & 1);
+                        const size_t j0 = h * d + even;
+                        const float x1 = x[j0] * inv * w[j0];
+                        const float x2 = x[j0 + 1] * inv * w[j0 + 1];
+                        const float c = cos_t[s * d + even];
+                        const float sn = sin_t[s * d + even + 1];
+                        o[p] = (p & 1) ? (x1 * sn + x2 * c) : (x1 * c - x2 * sn);
+                    }
+                }
+            }
+        }
+}
+
+/* C/wan/fuse.rs:321-342; C/rt/fuse/host.rs:93-96 (rms_factor), 217-241 (qk_norm),
+ * 247-276 (qk_rope_head, interleaved pairing) */
+void fvo_wan_qk_norm_rope16(const float* src, const float* w, const float* cos_t, const float* sin_t,
+                            float* out, size_t batch, size_t seq, size_t heads, size_t d,
+                            size_t src_width, size_t col_off, float eps) {
+    const size_t width = heads * d;
+    float* n = (float*)malloc(width * sizeof(float));
+    for (size_t b = 0; b < batch; b++)
+        for (size_t s = 0; s < seq; s++) {
+            const float* x = src + (b * seq + s) * src_width + col_off;
+            float ss = 0.0f;
+            for (size_t j = 0; j < width; j++) ss += x[j] * x[j];
+            const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+            for (size_t j = 0; j < width; j++) {
+                const float t = fvo_bf16_round(x[j] * inv);
+                n[j] = fvo_bf16_round(t * w[j]);
+            }
+            for (size_t h = 0; h < heads; h++) {
+                float* o = out + ((b * heads + h) * seq + s) * d;
+                const float* nh = n + h * d;
+                for (size_t p = 0; p < d; p++) {
+                    if (!cos_t || !sin_t) {
+                        o[p] = nh[p];   /* already rounded (round_weighted) */
+                    } else {
+                        const size_t even = p - (p & 1);
+                        const float x1 = nh[even], x2 = nh[even + 1];
+                        const float cv = cos_t[s * d + even], sv = sin_t[s * d + even + 1];
+                        o[p] = fvo_bf16_round((p & 1) ? (x2 * cv + x1 * sv) : (x1 * cv - x2 * sv));
+                    }
+                }
+            }
+        }
+    free(n);
+}
+
+/* C/rt/ops.rs:2352-2372 */
+void fvo_split_heads_bhsd(const float* src, float* out, size_t batch, size_t seq, size_t heads,
+                          size_t d, size_t src_width, size_t col_off) {
+    for (size_t b = 0; b < batch; b++)
+        for (size_t h = 0; h < heads; h++)
+            for (size_t s = 0; s < seq; s++)
+                memcpy(out + ((b * heads + h) * seq + s) * d,
+                       src + (b * seq + s) * src_width + col_off + h * d, d * sizeof(float));
+}
+
+/* C/rt/ops.rs:2374-2386 */
+void fvo_merge_heads(const float* src, float* out, size_t batch, size_t heads, size_t seq, size_t d) {
+    const size_t hd = heads * d;
+    for (size_t b = 0; b < batch; b++)
+        for (size_t s = 0; s < seq; s++)
+            for (size_t h = 0; h < heads; h++)
+                memcpy(out + (b * seq + s) * hd + h * d, src + ((b * heads + h) * seq + s) * d,
+                       d * sizeof(float));
+}

@@ -22,6 +22,13 @@
  *   fvo_topk_*            brute-force sort on small n, ties, -0.0, both orders
  *   fvo_vsa_tile_mean     closed form on constant/linear inputs
  *   fvo_shard_ranges      known answers C/rt/sp.rs:66-84
+ *   fvo_qk_norm_rope_bhsd / fvo_wan_qk_norm_rope16
+ *                         the two against each other within 0.03 on the closed-form
+ *                         inputs of C/wan/fuse.rs:627-663; no-rope == x*inv*w by hand;
+ *                         RMS of the normalised row == 1 for w == 1; the rotation keeps
+ *                         each pair's norm; rope with angle 0 == no rope
+ *   fvo_split_heads_bhsd / fvo_merge_heads
+ *                         brute-force index formula, merge(split(x)) == x
  */
 #ifndef FV_ORACLE_H
 #define FV_ORACLE_H
@@ -114,6 +121,27 @@ void fvo_vsa_coarse_scores(const float* qc, const float* kc, float* scores, size
 
 /* C/rt/sp.rs:16-28; out [world][2] = (start, len) */
 void fvo_shard_ranges(size_t seq, size_t world, size_t* out);
+
+/* ---- producer / consumer either side of the SDPA call --------------------------- */
+
+/* C/rt/ops.rs:2304-2350 (f32 op): RMSNorm of columns [col_off, col_off+heads*d) of each
+ * row of src [batch, seq, src_width] across all heads (sum of squares in index order),
+ * times w, optional interleaved RoPE (cos from the even slot, sin from the odd slot of
+ * the pair, tables [seq, d]; NULL tables = no rotation), out [batch, heads, seq, d]. */
+void fvo_qk_norm_rope_bhsd(const float* src, const float* w, const float* cos_t, const float* sin_t,
+                           float* out, size_t batch, size_t seq, size_t heads, size_t d,
+                           size_t src_width, size_t col_off, float eps);
+/* C/wan/fuse.rs:321-342 with C/rt/fuse/host.rs:217-270 under WAN_QK_NORM_ROPE
+ * (C/rt/fuse/policy.rs:404-412): bf16(bf16(x*inv)*w), rotation in f32, one rounding;
+ * values are bf16-representable f32. */
+void fvo_wan_qk_norm_rope16(const float* src, const float* w, const float* cos_t, const float* sin_t,
+                            float* out, size_t batch, size_t seq, size_t heads, size_t d,
+                            size_t src_width, size_t col_off, float eps);
+/* C/rt/ops.rs:2352-2372 */
+void fvo_split_heads_bhsd(const float* src, float* out, size_t batch, size_t seq, size_t heads,
+                          size_t d, size_t src_width, size_t col_off);
+/* C/rt/ops.rs:2374-2386 */
+void fvo_merge_heads(const float* src, float* out, size_t batch, size_t heads, size_t seq, size_t d);
 
 #ifdef __cplusplus
 }
