@@ -26,25 +26,39 @@ __global__ __launch_bounds__(256) void vsa_tile_mean_kernel(
     const int n = block_sizes[tile];
     const int* src = slot_src + (long)tile * kTileElems;
     float* ob = out + (bh * num_tiles + tile) * (long)dim;
+    auto load_tok = [&](long tok, int d0) -> f32x4 {
+        f32x4 v;
+        if constexpr (IN_BF16) {
+            const u32x2 raw = *reinterpret_cast<const u32x2*>(
+                (const uint16_t*)x + (bh * seq + tok) * dim + d0);
+            v[0] = __builtin_bit_cast(float, raw[0] << 16);
+            v[1] = __builtin_bit_cast(float, raw[0] & 0xffff0000u);
+            v[2] = __builtin_bit_cast(float, raw[1] << 16);
+            v[3] = __builtin_bit_cast(float, raw[1] & 0xffff0000u);
+        } else {
+            v = *reinterpret_cast<const f32x4*>((const float*)x + (bh * seq + tok) * dim + d0);
+            if (round16) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = bf16_bits_to_f32(bf16_rne_bits(v[e]));
+            }
+        }
+        return v;
+    };
     for (int d0 = ln * 4; d0 < dim; d0 += 128) {
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int j = 0; j < n; j++) {
-            const long tok = src[j];
-            f32x4 v;
-            if constexpr (IN_BF16) {
-                const u32x2 raw = *reinterpret_cast<const u32x2*>(
-                    (const uint16_t*)x + (bh * seq + tok) * dim + d0);
-                v[0] = __builtin_bit_cast(float, raw[0] << 16);
-                v[1] = __builtin_bit_cast(float, raw[0] & 0xffff0000u);
-                v[2] = __builtin_bit_cast(float, raw[1] << 16);
-                v[3] = __builtin_bit_cast(float, raw[1] & 0xffff0000u);
-            } else {
-                v = *reinterpret_cast<const f32x4*>((const float*)x + (bh * seq + tok) * dim + d0);
-                if (round16) {
+        int j = 0;
+        // eight loads in flight, then their adds in slot order (the order is the contract)
+        for (; j + 8 <= n; j += 8) {
+            f32x4 v[8];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) v[e] = bf16_bits_to_f32(bf16_rne_bits(v[e]));
-                }
-            }
+            for (int u = 0; u < 8; u++) v[u] = load_tok(src[j + u], d0);
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[e] = __fadd_rn(acc[e], v[u][e]);
+        }
+        for (; j < n; j++) {
+            const f32x4 v = load_tok(src[j], d0);
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[e] = __fadd_rn(acc[e], v[e]);
         }
@@ -106,9 +120,9 @@ __global__ __launch_bounds__(256) void vsa_coarse_scores_kernel(
 }
 
 // ---- coarse softmax x V (rt/vsa.rs:389-393, kernels/core.cu:177-252) ---------------
-// coarse[bh, qt, :] = softmax(scores[bh, qt, :]) vc[bh]; four query tiles per block
+// coarse[bh, qt, :] = softmax(scores[bh, qt, :]) vc[bh]; eight query tiles per block
 // share every vc row they read. dim = 128.
-constexpr int kCoarseRows = 4;
+constexpr int kCoarseRows = 8;
 __global__ __launch_bounds__(256) void vsa_coarse_pv_kernel(
     const float* __restrict__ scores, const float* __restrict__ vc, float* __restrict__ coarse,
     int nb) {
@@ -146,22 +160,33 @@ __global__ __launch_bounds__(256) void vsa_coarse_pv_kernel(
     __syncthreads();
     if (tid < rows) stat[tid] = 1.0f / (red[tid][0] + red[tid][1] + red[tid][2] + red[tid][3]);
     __syncthreads();
-    // each half-block owns two rows; lane d accumulates over all key tiles
+    // each half-block owns four rows; lane d accumulates over all key tiles, four vc rows
+    // in flight per step
+    constexpr int kOwn = kCoarseRows / 2;
     const int d = tid & 127, rh = tid >> 7;
     const float* vb = vc + bh * nb * 128L + d;
-    float a0 = 0.f, a1 = 0.f;
-    const float* p0 = p_lds + (2 * rh) * nb;
-    const float* p1 = p_lds + (2 * rh + 1) * nb;
-    const bool ok0 = 2 * rh < rows, ok1 = 2 * rh + 1 < rows;
-    if (ok0) {
-        for (int kt = 0; kt < nb; kt++) {
-            const float vv = vb[(long)kt * 128];
-            a0 += p0[kt] * vv;
-            if (ok1) a1 += p1[kt] * vv;
-        }
-        coarse[(bh * nb + q0 + 2 * rh) * 128L + d] = a0 * stat[2 * rh];
-        if (ok1) coarse[(bh * nb + q0 + 2 * rh + 1) * 128L + d] = a1 * stat[2 * rh + 1];
+    const float* pr = p_lds + (kOwn * rh) * nb;
+    float a[kOwn];
+#pragma unroll
+    for (int r = 0; r < kOwn; r++) a[r] = 0.f;
+    int kt = 0;
+    for (; kt + 4 <= nb; kt += 4) {
+        float vv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) vv[u] = vb[(long)(kt + u) * 128];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int r = 0; r < kOwn; r++) a[r] += pr[r * nb + kt + u] * vv[u];
     }
+    for (; kt < nb; kt++) {
+        const float vv = vb[(long)kt * 128];
+#pragma unroll
+        for (int r = 0; r < kOwn; r++) a[r] += pr[r * nb + kt] * vv;
+    }
+#pragma unroll
+    for (int r = 0; r < kOwn; r++)
+        if (kOwn * rh + r < rows) coarse[(bh * nb + q0 + kOwn * rh + r) * 128L + d] = a[r] * stat[kOwn * rh + r];
 }
 
 // ---- top-k (kernels/core.cu:576-619, kernels/attn3.cu:279-363) ----------------------
