@@ -31,9 +31,9 @@
 //     behind every MFMA that waits for the matrix pipe;
 //   * K/V tiles go global -> LDS directly (global_load_lds_dwordx4) into
 //     XOR-swizzled unpadded tiles, four buffers each;
-//   * workgroup ids are remapped so that the workgroups resident on one XCD
-//     walk consecutive query tiles of the same head (their K/V stream hits
-//     that XCD's L2).
+//   * dense launches remap workgroup ids so that the workgroups resident on one
+//     XCD walk consecutive query tiles of the same head (their K/V stream hits
+//     that XCD's L2); block-causal launches run longest tiles first.
 //
 // Time is counted in slots (one phase each); a phase covers a PAIR of key tiles
 // (128 keys): a matrix phase is 64 MFMAs (PV of the previous pair, QK of the
@@ -75,10 +75,24 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: branches on it stay scalar
     const int grp = wave >> 2;
     const int h = lane >> 5, c32 = lane & 31;
-    const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-    if (work >= p.total) return;
-    const int bh = work / p.nqt;
-    const int qt = CAUSAL ? (p.nqt - 1 - work % p.nqt) : (work % p.nqt);
+    // Work order. Dense (equal tiles): workgroup i runs on XCD i % 8, and XCD x takes the
+    // contiguous range [x, x+1) * per_xcd of (head, query tile) items, so its CUs stream one
+    // head's K/V through its L2 together. Block-causal (tiles differ in length by up to the
+    // whole band): longest first over the whole launch, tile index major and head minor;
+    // measured 9 % faster than the dense order, whose per-XCD ranges hold unequal work.
+    int bh, qt;
+    if constexpr (CAUSAL) {
+        const int work = blockIdx.x;
+        if (work >= p.total) return;
+        const int nbh = p.total / p.nqt;
+        bh = work % nbh;
+        qt = p.nqt - 1 - work / nbh;
+    } else {
+        const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
+        if (work >= p.total) return;
+        bh = work / p.nqt;
+        qt = work % p.nqt;
+    }
     const int q0 = qt * kPpBM;
     const int sq = p.sq, sk = p.sk;
     const int qlen = min(kPpBM, sq - q0);
