@@ -95,7 +95,7 @@ def test_declines(fv):
 
 @pytest.mark.parametrize("bt", [1560, 4680])
 def test_headline_causal_shape_sampled_rows(fv, oracle, bt):
-    """BASELINE config 3 at full size (21 frames x 1560 tokens) and the
+    """Self-Forcing frame-causal at full size (21 frames x 1560 tokens) and the
     reference's own 3-frame blocks; parity on sampled rows incl. frame edges."""
     import torch
 

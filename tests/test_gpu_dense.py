@@ -1,7 +1,7 @@
 """Parity of the gfx950 dense flash kernel (through the C ABI) against the CPU
 oracle's fp32 composed SDPA. Shapes follow the reference's flash_mma table
 (crates/fastvideo-gpucheck/src/kernels.rs:2286-2297, d = 128 rows) plus the
-BASELINE configs; tolerances: max|delta| <= 1e-2, cosine >= 0.9999 vs the fp32
+Wan-shaped benchmark configurations; tolerances: max|delta| <= 1e-2, cosine >= 0.9999 vs the fp32
 oracle on identical bf16-valued inputs, rel_l2 <= 1e-2 vs the oracle on the
 unrounded inputs, <= 2e-3 on rounded inputs (kernels.rs:2314-2328).
 """
@@ -21,7 +21,7 @@ SHAPES = [  # (bh, sq, sk, std)
     (2, 63, 4097, 1.0),
     (4, 1024, 1024, 2.0),
     (2, 2048, 2048, 1.0),
-    (12, 320, 320, 1.0),   # BASELINE config 1
+    (12, 320, 320, 1.0),   # tiny Wan-1.3B-shaped case
     (2, 128, 64, 1.0),
     (1, 129, 65, 1.0),
     (1, 127, 63, 1.0),
@@ -123,7 +123,7 @@ def test_declines(fv):
 
 
 def test_headline_shape_sampled_rows(fv, oracle):
-    """BASELINE config 2 at full size: S = 32760, H = 12; parity on sampled rows."""
+    """Wan-1.3B 480p self-attention at full size: S = 32760, H = 12; parity on sampled rows."""
     import torch
 
     bh, s, d = 12, 32760, 128

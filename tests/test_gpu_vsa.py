@@ -241,7 +241,7 @@ def test_declines_and_errors(fv):
 
 @pytest.mark.parametrize("grid,topk", [((32, 32, 32), 64), ((21, 30, 52), 125)])
 def test_headline_vsa_shapes(fv, oracle, grid, topk):
-    """BASELINE config 4 (512 full cubes, top-k 64 of 512) and the reference's own Wan
+    """The synthetic VSA benchmark geometry (512 full cubes, top-k 64 of 512) and the reference's own Wan
     480p geometry (624 tiles, top-k 125), H = 12, bf16: block index lists bit-exact at
     full size; fine + combine output checked on sampled query tiles."""
     import torch
