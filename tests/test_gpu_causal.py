@@ -23,6 +23,13 @@ CASES = [  # (bh, s, block_tokens, window, sink)
     (2, 96, 200, 0, 0),
     (2, 1000, 64, 2, 3),
     (1, 777, 100, 1, 0),
+    # band walks whose tile counts are odd / even and whose sink tiles are disjoint from the
+    # band (the pair-of-tiles phases round an odd count up with a fully masked tile)
+    (1, 1280, 64, 2, 1),    # window 2 blocks of one tile, one sink tile: 3-tile walks
+    (1, 1280, 128, 1, 1),
+    (2, 1500, 192, 2, 2),
+    (1, 2049, 256, 3, 0),
+    (1, 900, 300, 0, 0),
 ]
 
 

@@ -62,6 +62,23 @@ def test_dense_matches_composed_oracle(fv, oracle, bh, sq, sk, std):
     assert np.array_equal(got16, oracle.quantize_bf16(got))
 
 
+@pytest.mark.parametrize("sk", [1, 2, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 383, 449, 511, 513])
+def test_every_tile_count_parity_and_key_tail(fv, oracle, sk):
+    """The kernel walks the keys two 64-key tiles per phase: odd and even tile counts,
+    full and ragged last tiles, one to nine tiles; query tails on both sides of a
+    256-query workgroup."""
+    import torch
+
+    d, bh = 128, 2
+    for sq in (1, 259):
+        announce(f"dense tile-count sweep bh={bh} sq={sq} sk={sk}")
+        q, k, v = qkv(5000 + sk, bh, sq, sk, d, 1.0)
+        want = oracle.sdpa_composed(q, k, v)
+        got = fv.sdpa_dense_bf16(*(to_dev_bf16(x) for x in (q, k, v)), out_bf16=False)
+        torch.cuda.synchronize()
+        assert_parity(got.cpu().numpy(), want, f"dense_sweep_{sq}x{sk}")
+
+
 def test_dense_vs_unrounded_f32_inputs(fv, oracle):
     import torch
 
