@@ -97,6 +97,14 @@ def bench_vsa(args):
         "fine": timed(lambda: V.vsa_fine(qt, kt, vt, sel, ctx, scale), 10, 2)[2],
         "combine": timed(lambda: V.vsa_combine(sparse, coarse, gate, ctx, out=out), 10, 2)[2],
     }
+    # the fine kernel alone on the selection the reference's own fine-kernel benchmark uses
+    # (gpucheck kernels_attn.rs:199-208): tile (i + 7h + j) mod nb for j < topk, i.e. a band of
+    # consecutive key tiles that neighbouring query tiles share almost entirely
+    ii = torch.arange(nb, device=dev).view(1, nb, 1)
+    hh = torch.arange(h, device=dev).view(h, 1, 1)
+    jj = torch.arange(topk, device=dev).view(1, 1, topk)
+    sel_band = ((ii + 7 * hh + jj) % nb).to(torch.int32).contiguous()
+    stages["fine_banded_selection"] = timed(lambda: V.vsa_fine(qt, kt, vt, sel_band, ctx, scale), 10, 2)[2]
     flops = 4.0 * (h * nb * 64) * (topk * 64) * d
     fine_tflops = flops / (stages["fine"] * 1e-3) / 1e12
     rec = {
@@ -110,7 +118,8 @@ def bench_vsa(args):
         "stages_median_ms": {k2: round(v2, 4) for k2, v2 in stages.items()},
         "roofline": {"bound": "mfma", "achieved": round(fine_tflops, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(fine_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::vsa_fine_kernel",
-                     "avg_kernel_ms": round(stages["fine"], 4)},
+                     "avg_kernel_ms": round(stages["fine"], 4),
+                     "banded_selection_tflops": round(flops / (stages["fine_banded_selection"] * 1e-3) / 1e12, 3)},
     }
     print(json.dumps(rec), flush=True)
 
