@@ -300,14 +300,11 @@ extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 
 extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal,
                                                hipStream_t stream) {
-    static bool attr_done[2] = {false, false};
+    static std::atomic<unsigned long long> attr_done[2];
     const void* fn = causal ? (const void*)fv::flash_fwd_pp2_d128<true> : (const void*)fv::flash_fwd_pp2_d128<false>;
     const int lds = fv::kPp2LdsBytes;
-    if (!attr_done[causal ? 1 : 0]) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return e;
-        attr_done[causal ? 1 : 0] = true;
-    }
+    hipError_t e = fv_set_max_lds_once(fn, lds, attr_done[causal ? 1 : 0]);
+    if (e != hipSuccess) return e;
     const dim3 grid(p->per_xcd * 8), block(512);
     if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp2_d128<true>, grid, block, lds, stream, *p);
     else hipLaunchKernelGGL(fv::flash_fwd_pp2_d128<false>, grid, block, lds, stream, *p);

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace fv {
 
 struct FlashParams {
@@ -62,3 +64,17 @@ extern "C" hipError_t fv_internal_launch_combine(const float* sparse, const floa
 int fv_fail_hip(hipError_t e, const char* what);   // returns -(int)e
 int fv_decline(const char* why);                    // returns FV_DECLINED
 int fv_invalid(const char* why);                    // returns -(int)hipErrorInvalidValue
+
+// Raise a kernel's dynamic LDS limit once per device (the attribute belongs to the function
+// on the current device). `done` holds one bit per device ordinal; concurrent first calls may
+// both set the attribute, which is harmless.
+inline hipError_t fv_set_max_lds_once(const void* fn, int bytes, std::atomic<unsigned long long>& done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}

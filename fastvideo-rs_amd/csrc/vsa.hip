@@ -492,13 +492,10 @@ extern "C" hipError_t fv_internal_launch_coarse(const float* qc, const float* kc
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || !coarse) return e;
     const size_t lds = sizeof(float) * kCoarseRows * (size_t)nb;
-    static bool attr_done = false;
-    if (!attr_done) {
-        e = hipFuncSetAttribute((const void*)vsa_coarse_pv_kernel,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, sizeof(float) * kCoarseRows * kTopkMaxN);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static std::atomic<unsigned long long> attr_done;
+    e = fv_set_max_lds_once((const void*)vsa_coarse_pv_kernel, (int)(sizeof(float) * kCoarseRows * kTopkMaxN),
+                            attr_done);
+    if (e != hipSuccess) return e;
     const dim3 g2((nb + kCoarseRows - 1) / kCoarseRows, (unsigned)bh);
     hipLaunchKernelGGL(vsa_coarse_pv_kernel, g2, dim3(256), lds, st, scores, vc, coarse, nb);
     return hipGetLastError();
