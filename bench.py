@@ -8,7 +8,7 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny|vsa624|vsa512|prep) are for the
+Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vsa624|vsa512|prep) are for the
 design notes; the driver's line is the default `self`.
 """
 import argparse
@@ -36,6 +36,7 @@ WORKLOADS = {
     "c5": (40, 75600, 75600, 0, "Wan2.1-14B 720p self-attention, B=1 H=40 S=75600 d=128 bf16"),
     "c5cross": (40, 75600, 512, 0, "Wan2.1-14B 720p cross-attention, H=40 Sq=75600 Sk=512"),
     "tiny": (12, 320, 320, 0, "tiny Wan-1.3B-shaped self-attention, H=12 S=320 d=128"),
+    "self_d64": (24, 32760, 32760, 0, "head dim 64 self-attention, B=1 H=24 S=32760 d=64 bf16 non-causal"),
 }
 
 
@@ -268,7 +269,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     h, sq, sk, bt, desc = WORKLOADS[args.workload]
-    d = 128
+    d = 64 if args.workload.endswith("_d64") else 128
     g = torch.Generator(device=dev).manual_seed(20240)
     q = torch.randn((h, sq, d), generator=g, device=dev).to(torch.bfloat16)
     k = torch.randn((h, sk, d), generator=g, device=dev).to(torch.bfloat16)
@@ -338,7 +339,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.out_bf16 else None,
-                     "kernel": "fv::flash_fwd_pp2_d128<true>" if bt else "fv::flash_fwd_pp2_d128<false>",
+                     "kernel": f"fv::flash_fwd_pp2<{'true' if bt else 'false'}, {d}>",
                      "avg_kernel_ms": round(avg_kernel_ms, 4), "median_kernel_ms": round(kern_ms[len(kern_ms) // 2], 4),
                      "min_hbm_bytes": bytes_min,
                      "hbm_frac_at_min_traffic": round(bytes_min / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},

@@ -17,7 +17,28 @@ namespace fv {
 
 constexpr int kTileRows = 64;
 constexpr int kRowBytes = 256;
-constexpr int kTileBytes = kTileRows * kRowBytes;   // 16 KB
+constexpr int kTileBytes = kTileRows * kRowBytes;   // 16 KB (head dim 128)
+
+// Tile geometry by head dim D (128 or 64): rows of 2 D bytes, 16-byte chunks, and the XOR
+// swizzles that make the operand reads bank-conflict free.
+//   D = 128 (256 B rows, 16 chunks): K chunk ^ (row & 15); V chunk ^ ((row & 3) << 2).
+//   D = 64  (128 B rows,  8 chunks): two rows share a 256 B bank line, so the K swizzle
+//     advances every second row, chunk ^ ((row >> 1) & 7), and the V swizzle separates
+//     rows j and j+2 of a transposed 4-row read, chunk ^ (((row >> 1) & 1) << 2).
+template <int D>
+struct TileGeo {
+    static_assert(D == 128 || D == 64, "head dim 128 or 64");
+    static constexpr int kRow = 2 * D;                   // bytes per row
+    static constexpr int kTile = kTileRows * kRow;       // bytes per tile
+    static constexpr int kChunks = kRow / 16;            // 16-byte chunks per row
+    static constexpr int kRowsPerDma = 1024 / kRow;      // rows one wave-wide DMA instruction covers
+    static constexpr int kDmaPerTile = kTile / 1024;
+    static constexpr int kVGroups = D / 16;              // PV groups per tile (2 MFMAs each)
+    static constexpr int kKGroups = D / 16;              // QK groups per tile
+    static constexpr int kGroups = kVGroups + kKGroups;
+    static FV_DEV int kswz(int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); }
+    static FV_DEV int vswz(int r) { return D == 128 ? ((r & 3) << 2) : (((r >> 1) & 1) << 2); }
+};
 
 typedef __attribute__((address_space(1))) void glb_void;
 typedef __attribute__((address_space(3))) void lds_void;
@@ -69,22 +90,24 @@ FV_DEV void lds_dma16_s(unsigned lds_base, const void* sbase_in, unsigned voff) 
         : "memory");
 }
 
-// Per-lane source offsets of the tile loads, computed once per kernel: with NW
-// waves sharing a 64-row tile a wave issues ITER = 16 / NW instructions of 4 rows
-// each; instruction `it` of wave w covers rows (w*ITER + it)*4 .. +3, lane i
-// fetching the 16 B chunk that belongs at position i%16 of row + i/16.
-template <int NW>
+// Per-lane source offsets of the tile loads, computed once per kernel: a wave-wide
+// DMA instruction moves 1 KB = 4 rows of 256 B (D = 128) or 8 rows of 128 B (D = 64);
+// with NW waves sharing a 64-row tile a wave issues ITER = (tile KB) / NW of them;
+// lane i fetches the 16 B chunk that belongs at its position of its row.
+template <int NW, int D = 128>
 struct TileDma {
-    static constexpr int ITER = 16 / NW;
+    using G = TileGeo<D>;
+    static constexpr int ITER = G::kDmaPerTile / NW;
+    static_assert(ITER >= 1, "more waves than DMA instructions per tile");
     unsigned koff[ITER];   // byte offset from the tile's first row, K swizzle
     unsigned voff[ITER];   // same, V swizzle
     FV_DEV void init(int wave, int lane) {
-        const int p = lane & 15;
+        const int p = lane % G::kChunks;
 #pragma unroll
         for (int it = 0; it < ITER; it++) {
-            const int r = (wave * ITER + it) * 4 + (lane >> 4);
-            koff[it] = r * kRowBytes + ((p ^ (r & 15)) << 4);
-            voff[it] = r * kRowBytes + ((p ^ ((r & 3) << 2)) << 4);
+            const int r = (wave * ITER + it) * G::kRowsPerDma + lane / G::kChunks;
+            koff[it] = r * G::kRow + ((p ^ G::kswz(r)) << 4);
+            voff[it] = r * G::kRow + ((p ^ G::vswz(r)) << 4);
         }
     }
     // A tile load prepared ahead of its issue: everything the DMA instructions need,
@@ -98,20 +121,20 @@ struct TileDma {
     FV_DEV Prepared prepare(lds_u8* buf, const uint16_t* tile_base, int rows_valid, int wave) const {
         Prepared d;
         d.base = (unsigned long long)tile_base;
-        d.lds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 4 * kRowBytes);
+        d.lds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 1024);
 #pragma unroll
         for (int it = 0; it < ITER; it++) d.off[it] = IS_V ? voff[it] : koff[it];
         if (rows_valid < kTileRows) {
 #pragma unroll
             for (int it = 0; it < ITER; it++) {
-                const int over = max(0, (int)(d.off[it] >> 8) - (rows_valid - 1));
-                d.off[it] -= over * kRowBytes;
+                const int over = max(0, (int)(d.off[it] / G::kRow) - (rows_valid - 1));
+                d.off[it] -= over * G::kRow;
             }
         }
         return d;
     }
     static FV_DEV void issue_prepared(const Prepared& d, int it) {
-        lds_dma16_s(d.lds + it * 4 * kRowBytes, (const void*)d.base, d.off[it]);
+        lds_dma16_s(d.lds + it * 1024, (const void*)d.base, d.off[it]);
     }
     // The same without per-descriptor lane offsets (scalars only): the tail clamp, needed by
     // the last key tile alone, is then taken at issue time behind a wave-uniform branch.
@@ -123,7 +146,7 @@ struct TileDma {
     FV_DEV Target target(lds_u8* buf, const uint16_t* tile_base, int rows_valid, int wave) const {
         Target d;
         d.base = (unsigned long long)tile_base;
-        d.lds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 4 * kRowBytes);
+        d.lds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 1024);
         d.rows_valid = rows_valid;
         return d;
     }
@@ -132,13 +155,13 @@ struct TileDma {
         if (d.rows_valid >= kTileRows) {
 #pragma unroll
             for (int it = 0; it < ITER; it++)
-                lds_dma16_s(d.lds + it * 4 * kRowBytes, (const void*)d.base, IS_V ? voff[it] : koff[it]);
+                lds_dma16_s(d.lds + it * 1024, (const void*)d.base, IS_V ? voff[it] : koff[it]);
         } else {
 #pragma unroll
             for (int it = 0; it < ITER; it++) {
                 const unsigned off = IS_V ? voff[it] : koff[it];
-                const int over = max(0, (int)(off >> 8) - (d.rows_valid - 1));
-                lds_dma16_s(d.lds + it * 4 * kRowBytes, (const void*)d.base, off - over * kRowBytes);
+                const int over = max(0, (int)(off / G::kRow) - (d.rows_valid - 1));
+                lds_dma16_s(d.lds + it * 1024, (const void*)d.base, off - over * G::kRow);
             }
         }
     }
@@ -147,17 +170,17 @@ struct TileDma {
     // content only has to be finite data the tensor already holds.
     template <bool IS_V>
     FV_DEV void issue(lds_u8* buf, const uint16_t* tile_base, int rows_valid, int wave) const {
-        const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 4 * kRowBytes);
+        const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 1024);
         if (rows_valid >= kTileRows) {
 #pragma unroll
             for (int it = 0; it < ITER; it++)
-                lds_dma16_s(base + it * 4 * kRowBytes, tile_base, IS_V ? voff[it] : koff[it]);
+                lds_dma16_s(base + it * 1024, tile_base, IS_V ? voff[it] : koff[it]);
         } else {
 #pragma unroll
             for (int it = 0; it < ITER; it++) {
                 const unsigned off = IS_V ? voff[it] : koff[it];
-                const int over = max(0, (int)(off >> 8) - (rows_valid - 1));
-                lds_dma16_s(base + it * 4 * kRowBytes, tile_base, off - over * kRowBytes);
+                const int over = max(0, (int)(off / G::kRow) - (rows_valid - 1));
+                lds_dma16_s(base + it * 1024, tile_base, off - over * G::kRow);
             }
         }
     }
@@ -190,14 +213,18 @@ struct TileReadBases {
     int k;   // K A-operand: ^ (dk << 5), + kb * 32 rows
     int v;   // V^T A-operand (transposed read): ^ (db << 6), + (16 t + 8 g) rows
 };
+template <int D = 128>
 FV_DEV TileReadBases tile_read_bases(int lane) {
+    using G = TileGeo<D>;
     const int h = lane >> 5, c32 = lane & 31;
     const int b16 = lane >> 4, i16 = lane & 15;
     TileReadBases b;
-    b.k = c32 * kRowBytes + ((((c32 & 15) ^ h)) << 4);
+    // K: lane reads logical chunk 2 dk + h of row c32 (+32): physical (2 dk + h) ^ kswz(row)
+    b.k = c32 * G::kRow + ((G::kswz(c32) ^ h) << 4);
+    // V^T: lane reads 8 bytes at d = 32 db + 16 (b16 & 1) + 4 (i16 & 3) of row 4 h + i16/4 (+16 t, +8)
     const int r = 4 * h + (i16 >> 2);
     const int c_lane = 2 * (b16 & 1) + ((i16 & 3) >> 1);
-    b.v = r * kRowBytes + ((((i16 >> 2) << 2) + c_lane) << 4) + 8 * (i16 & 1);
+    b.v = r * G::kRow + ((G::vswz(r) ^ c_lane) << 4) + 8 * (i16 & 1);
     return b;
 }
 
@@ -274,7 +301,8 @@ FV_DEV void softmax_tile(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float
 }
 
 // softmax_tile over a pair of tiles (128 keys) with one shared max / rescale decision.
-FV_DEV void softmax_tile_pair(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxState& st, f32x16 (&o)[4],
+template <int NO = 4>
+FV_DEV void softmax_tile_pair(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxState& st, f32x16 (&o)[NO],
                               float sl2, bf16x8 (&pb0)[4], bf16x8 (&pb1)[4]) {
     const float NEG = neg_inf();
     float mx = s0[0][0];
@@ -295,7 +323,7 @@ FV_DEV void softmax_tile_pair(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxState& st
         const float alpha = (st.m_used == NEG) ? 0.f : fast_exp2(st.ms_used - ms_new);
         st.l_acc *= alpha;
 #pragma unroll
-        for (int db = 0; db < 4; db++)
+        for (int db = 0; db < NO; db++)
 #pragma unroll
             for (int i = 0; i < 16; i++) o[db][i] *= alpha;
         st.m_used = st.m_run;
@@ -324,14 +352,16 @@ FV_DEV void softmax_tile_pair(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxState& st
 }
 
 // O^T (128 d x 32 queries) += V^T P^T.
-FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 (&o)[4]) {
+template <int D = 128>
+FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 (&o)[D / 32]) {
+    constexpr int kRow = TileGeo<D>::kRow;
 #pragma unroll
     for (int t = 0; t < 4; t++) {
 #pragma unroll
-        for (int db = 0; db < 4; db++) {
-            const int a0 = (v_base ^ (db << 6)) + (16 * t) * kRowBytes;
+        for (int db = 0; db < D / 32; db++) {
+            const int a0 = (v_base ^ (db << 6)) + (16 * t) * kRow;
             const s16x4 lo = lds_read_tr16_b64(vb + a0);
-            const s16x4 hi = lds_read_tr16_b64(vb + a0 + 8 * kRowBytes);
+            const s16x4 hi = lds_read_tr16_b64(vb + a0 + 8 * kRow);
             s16x8 a;
             a.lo = lo;
             a.hi = hi;
@@ -348,34 +378,37 @@ FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 
 // matrix-pipe time earlier instead of on LDS latency plus the 64 B/clk per-SIMD
 // LDS return path. sched_barrier keeps the compiler from re-serialising reads
 // behind MFMAs.
-template <bool DO_PV, int kAhead, class Hook>
+template <bool DO_PV, int kAhead, class Hook, int D = 128>
 FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& rb,
-                       const bf16x8 (&pb)[4], f32x16 (&o)[4], const bf16x8 (&qf)[8],
+                       const bf16x8 (&pb)[4], f32x16 (&o)[D / 32], const bf16x8 (&qf)[D / 16],
                        f32x16 (&s)[2], Hook&& hook) {
-    constexpr int G0 = DO_PV ? 0 : 8;
-    bf16x8 f[16][2];
+    using G = TileGeo<D>;
+    constexpr int NV = G::kVGroups, NG = G::kGroups;
+    constexpr int G0 = DO_PV ? 0 : NV;
+    constexpr int kPerT = D / 64;   // V groups per 16-key group t (each covers two 32-wide d blocks)
+    bf16x8 f[NG][2];
     auto issue = [&](int g) {
-        if (g < 8) {          // V^T fragments: key group t = g/2, d blocks 2*(g%2), 2*(g%2)+1
+        if (g < NV) {         // V^T fragments: key group t, d blocks 2*(g % kPerT) + {0, 1}
 #pragma unroll
             for (int x = 0; x < 2; x++) {
-                const int t = g >> 1, db = 2 * (g & 1) + x;
-                const int a0 = (rb.v ^ (db << 6)) + (16 * t) * kRowBytes;
+                const int t = g / kPerT, db = 2 * (g % kPerT) + x;
+                const int a0 = (rb.v ^ (db << 6)) + (16 * t) * G::kRow;
                 s16x8 a;
                 a.lo = lds_read_tr16_b64(vb + a0);
-                a.hi = lds_read_tr16_b64(vb + a0 + 8 * kRowBytes);
+                a.hi = lds_read_tr16_b64(vb + a0 + 8 * G::kRow);
                 f[g][x] = __builtin_bit_cast(bf16x8, a);
             }
-        } else {              // K fragments: d chunk dk = g-8, key blocks 0 and 1
+        } else {              // K fragments: d chunk dk = g - NV, key blocks 0 and 1
 #pragma unroll
             for (int x = 0; x < 2; x++)
-                f[g][x] = lds_read_b128(kb + (rb.k ^ ((g - 8) << 5)) + x * 32 * kRowBytes);
+                f[g][x] = lds_read_b128(kb + (rb.k ^ ((g - NV) << 5)) + x * 32 * G::kRow);
         }
     };
     auto run = [&](int g) {
-        if (g < 8) {
+        if (g < NV) {
 #pragma unroll
             for (int x = 0; x < 2; x++) {
-                const int t = g >> 1, db = 2 * (g & 1) + x;
+                const int t = g / kPerT, db = 2 * (g % kPerT) + x;
                 o[db] = mfma32(f[g][x], pb[t], o[db]);
             }
         } else {
@@ -383,14 +416,14 @@ FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& 
                                  0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int x = 0; x < 2; x++)   // S is born at dk == 0, not before the PV part
-                s[x] = mfma32(f[g][x], qf[g - 8], g == 8 ? zero : s[x]);
+                s[x] = mfma32(f[g][x], qf[g - NV], g == NV ? zero : s[x]);
         }
     };
 #pragma unroll
-    for (int g = G0; g < G0 + kAhead && g < 16; g++) issue(g);
+    for (int g = G0; g < G0 + kAhead && g < NG; g++) issue(g);
 #pragma unroll
-    for (int g = G0; g < 16; g++) {
-        if (g + kAhead < 16) issue(g + kAhead);
+    for (int g = G0; g < NG; g++) {
+        if (g + kAhead < NG) issue(g + kAhead);
         __builtin_amdgcn_sched_barrier(0);
         run(g);
         __builtin_amdgcn_sched_barrier(0);
@@ -400,10 +433,11 @@ FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& 
 
 // Q^T fragments for the wave's 32 queries: rows row0 + lane%32 of a row-major
 // [rows][128] bf16 tensor; rows >= nrows read as zero.
-FV_DEV void load_q_frags(const uint16_t* q, int row, bool ok, int lane, bf16x8 (&qf)[8]) {
-    const uint16_t* src = q + (size_t)row * 128 + 8 * (lane >> 5);
+template <int D = 128>
+FV_DEV void load_q_frags(const uint16_t* q, int row, bool ok, int lane, bf16x8 (&qf)[D / 16]) {
+    const uint16_t* src = q + (size_t)row * D + 8 * (lane >> 5);
 #pragma unroll
-    for (int dk = 0; dk < 8; dk++) {
+    for (int dk = 0; dk < D / 16; dk++) {
         u32x4 t = {0u, 0u, 0u, 0u};
         if (ok) t = *reinterpret_cast<const u32x4*>(src + 16 * dk);
         qf[dk] = __builtin_bit_cast(bf16x8, t);

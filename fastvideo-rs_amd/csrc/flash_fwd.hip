@@ -1,4 +1,4 @@
-// Dense and block-causal flash attention forward for gfx950, head_dim 128, bf16.
+// Dense and block-causal flash attention forward for gfx950, head dim 128 or 64, bf16.
 //
 // Replaces the reference's flash_mma_fwd2_d128 / flash_mma_fwd2_causal_d128
 // (crates/fastvideo-cudarc/src/rt/kernels/attn2.cu:40-352) behind
@@ -58,16 +58,15 @@
 
 namespace fv {
 
-constexpr int kD = 128;          // head dim
 constexpr int kBN = 64;          // keys per tile
-
 constexpr int kPpBM = 256;      // queries per workgroup
+constexpr int kRing2 = 4;        // K buffers = V buffers: 128 KB of LDS at D = 128, 64 KB at D = 64
 
-constexpr int kRing2 = 4;
-constexpr int kPp2LdsBytes = 2 * kRing2 * kTileBytes;   // K[4], V[4] = 128 KB
-
-template <bool CAUSAL>
-__global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p) {
+template <bool CAUSAL, int D>
+__global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
+    using G = TileGeo<D>;
+    constexpr int kD = D;
+    constexpr int kTileBytes = G::kTile;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     lds_u8* smem = (lds_u8*)smem_raw;
 
@@ -140,41 +139,46 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
     auto kbuf = [&](int t) -> lds_u8* { return smem + (t & (kRing2 - 1)) * kTileBytes; };
     auto vbuf = [&](int t) -> lds_u8* { return smem + (kRing2 + (t & (kRing2 - 1))) * kTileBytes; };
 
-    TileDma<8> dma;
+    TileDma<8, D> dma;
     dma.init(wave, lane);
     // tiles past the end repeat the last one
     auto target_k = [&](int t) {
         const int kv0 = kv0_of(t);
-        return dma.prepare<false>(kbuf(t), Kh + (size_t)kv0 * kD, sk - kv0, wave);
+        return dma.template prepare<false>(kbuf(t), Kh + (size_t)kv0 * kD, sk - kv0, wave);
     };
     auto target_v = [&](int t) {
         const int kv0 = kv0_of(t);
-        return dma.prepare<true>(vbuf(t), Vh + (size_t)kv0 * kD, sk - kv0, wave);
+        return dma.template prepare<true>(vbuf(t), Vh + (size_t)kv0 * kD, sk - kv0, wave);
     };
+    using Dma = TileDma<8, D>;
+    constexpr int kIt = Dma::ITER;   // DMA instructions per wave and tile: 2 (D = 128) or 1 (D = 64)
     {
-        const TileDma<8>::Prepared a0 = target_k(0), a1 = target_k(1);
-        TileDma<8>::issue_prepared(a0, 0);
-        TileDma<8>::issue_prepared(a0, 1);
-        TileDma<8>::issue_prepared(a1, 0);
-        TileDma<8>::issue_prepared(a1, 1);
-    }
-    {   // zero V buffers 2 and 3: 32 KB, 64 B per thread
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        lds_u8* zb = smem + (kRing2 + 2) * kTileBytes + tid * 64;
+        const typename Dma::Prepared a0 = target_k(0), a1 = target_k(1);
 #pragma unroll
-        for (int i = 0; i < 4; i++) lds_write_b128(zb + 16 * i, z);
+        for (int it = 0; it < kIt; it++) {
+            Dma::issue_prepared(a0, it);
+            Dma::issue_prepared(a1, it);
+        }
     }
-    bf16x8 qf[8];
+    {   // zero V buffers 2 and 3 (two tiles), an equal share per thread
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        constexpr int kPer = 2 * kTileBytes / 512;
+        lds_u8* zb = smem + (kRing2 + 2) * kTileBytes + tid * kPer;
+#pragma unroll
+        for (int i = 0; i < kPer / 16; i++) lds_write_b128(zb + 16 * i, z);
+    }
+    bf16x8 qf[D / 16];
     {
         const int row = wave * 32 + c32;
-        load_q_frags(Qh, row, row < qlen, lane, qf);   // drains vmcnt: K(0), K(1) have landed too
+        load_q_frags<D>(Qh, row, row < qlen, lane, qf);   // drains vmcnt: K(0), K(1) have landed too
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the zero fill is in LDS
-    const TileReadBases rb = tile_read_bases(lane);
+    const TileReadBases rb = tile_read_bases<D>(lane);
 
-    f32x16 o[4];
+    constexpr int kNO = D / 32;   // 32-wide d blocks of the accumulator
+    f32x16 o[kNO];
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < kNO; db++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o[db][i] = 0.f;
     SoftmaxState st;
@@ -189,7 +193,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
             pb1[t][x] = (__bf16)0.0f;
         }
 
-    TileDma<8>::Prepared dk0 = target_k(2), dk1 = target_k(3), dv0 = target_v(0), dv1 = target_v(1);
+    typename Dma::Prepared dk0 = target_k(2), dk1 = target_k(3), dv0 = target_v(0), dv1 = target_v(1);
 
     block_barrier();                 // K(0), K(1), zeros resident
     if (grp == 1) block_barrier();   // group 1 idles through slot 0
@@ -230,18 +234,32 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
         // ---- matrix phase: group 0 in slot 2m, group 1 in slot 2m+1 ----
         __builtin_amdgcn_s_setprio(1);
         constexpr int kAhead = CAUSAL ? 2 : 3;
-        mfma_phase<true, kAhead>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, [&](int g) {
-            if (g == 1) TileDma<8>::issue_prepared(dk0, 0);
-            if (g == 2) TileDma<8>::issue_prepared(dk0, 1);
-            if (g == 4) TileDma<8>::issue_prepared(dk1, 0);
-            if (g == 5) TileDma<8>::issue_prepared(dk1, 1);
-        });
-        mfma_phase<true, kAhead>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, [&](int g) {
-            if (g == 1) TileDma<8>::issue_prepared(dv0, 0);
-            if (g == 2) TileDma<8>::issue_prepared(dv0, 1);
-            if (g == 4) TileDma<8>::issue_prepared(dv1, 0);
-            if (g == 5) TileDma<8>::issue_prepared(dv1, 1);
-        });
+        // DMA issue slots: after groups 1, 2 (first tile of the pair) and 4, 5 (second) at
+        // D = 128; after groups 1 and 3 at D = 64 (one instruction per tile and wave)
+        auto hook_k = [&](int g) {
+            if constexpr (kIt == 2) {
+                if (g == 1) Dma::issue_prepared(dk0, 0);
+                if (g == 2) Dma::issue_prepared(dk0, 1);
+                if (g == 4) Dma::issue_prepared(dk1, 0);
+                if (g == 5) Dma::issue_prepared(dk1, 1);
+            } else {
+                if (g == 1) Dma::issue_prepared(dk0, 0);
+                if (g == 3) Dma::issue_prepared(dk1, 0);
+            }
+        };
+        auto hook_v = [&](int g) {
+            if constexpr (kIt == 2) {
+                if (g == 1) Dma::issue_prepared(dv0, 0);
+                if (g == 2) Dma::issue_prepared(dv0, 1);
+                if (g == 4) Dma::issue_prepared(dv1, 0);
+                if (g == 5) Dma::issue_prepared(dv1, 1);
+            } else {
+                if (g == 1) Dma::issue_prepared(dv0, 0);
+                if (g == 3) Dma::issue_prepared(dv1, 0);
+            }
+        };
+        mfma_phase<true, kAhead, decltype(hook_k)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_k);
+        mfma_phase<true, kAhead, decltype(hook_v)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_v);
         __builtin_amdgcn_s_setprio(0);
         wait_vmcnt<0>();             // this wave's loads of this phase have landed
         __builtin_amdgcn_sched_barrier(0);
@@ -250,7 +268,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
         // ---- VALU phase: group 0 in slot 2m+1, group 1 in slot 2m+2 ----
         mask_tile(s0, 2 * m);
         mask_tile(s1, 2 * m + 1);
-        softmax_tile_pair(s0, s1, st, o, sl2, pb0, pb1);
+        softmax_tile_pair<kNO>(s0, s1, st, o, sl2, pb0, pb1);
         // P and the row sum must be complete before the barrier: without this the
         // compiler sinks the exponentials past it, into the matrix phase
         asm volatile("" ::"v"(pb0[0]), "v"(pb0[1]), "v"(pb0[2]), "v"(pb0[3]), "v"(pb1[0]), "v"(pb1[1]),
@@ -266,8 +284,8 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
         }
     }
     // O += P V of the last pair (their V landed before the last barrier both groups passed)
-    pv_tile(vbuf(2 * np - 2), rb.v, pb0, o);
-    pv_tile(vbuf(2 * np - 1), rb.v, pb1, o);
+    pv_tile<D>(vbuf(2 * np - 2), rb.v, pb0, o);
+    pv_tile<D>(vbuf(2 * np - 1), rb.v, pb1, o);
 
     const float l_tot = pair_sum(st.l_acc);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
@@ -275,7 +293,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
     if (row < qlen) {
         const size_t base = ((size_t)bh * sq + q0 + row) * kD;
 #pragma unroll
-        for (int db = 0; db < 4; db++)
+        for (int db = 0; db < kNO; db++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int d0 = 32 * db + 8 * g + 4 * h;
@@ -298,15 +316,21 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2_d128(const FlashParams p
 
 extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 
-extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal,
-                                               hipStream_t stream) {
-    static std::atomic<unsigned long long> attr_done[2];
-    const void* fn = causal ? (const void*)fv::flash_fwd_pp2_d128<true> : (const void*)fv::flash_fwd_pp2_d128<false>;
-    const int lds = fv::kPp2LdsBytes;
-    hipError_t e = fv_set_max_lds_once(fn, lds, attr_done[causal ? 1 : 0]);
+namespace {
+template <bool CAUSAL, int D>
+hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
+    static std::atomic<unsigned long long> attr_done;
+    constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
+    hipError_t e = fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<CAUSAL, D>, lds, attr_done);
     if (e != hipSuccess) return e;
-    const dim3 grid(p->per_xcd * 8), block(512);
-    if (causal) hipLaunchKernelGGL(fv::flash_fwd_pp2_d128<true>, grid, block, lds, stream, *p);
-    else hipLaunchKernelGGL(fv::flash_fwd_pp2_d128<false>, grid, block, lds, stream, *p);
+    hipLaunchKernelGGL((fv::flash_fwd_pp2<CAUSAL, D>), dim3(p->per_xcd * 8), dim3(512), lds, stream, *p);
     return hipGetLastError();
+}
+}  // namespace
+
+extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal, int d,
+                                               hipStream_t stream) {
+    if (d == 128) return causal ? launch_flash<true, 128>(p, stream) : launch_flash<false, 128>(p, stream);
+    if (d == 64) return causal ? launch_flash<true, 64>(p, stream) : launch_flash<false, 64>(p, stream);
+    return hipErrorInvalidValue;
 }

@@ -87,8 +87,8 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
         // (the reference asserts that identity for its own kernels, gpucheck kernels_wan.rs:230-261).
         if (block_tokens >= sq && block_tokens >= sk) causal = false;
     }
-    hipError_t e = fv_internal_launch_flash(&p, causal ? 1 : 0, (hipStream_t)stream);
-    if (e != hipSuccess) return fail_hip(e, causal ? "flash_fwd_pp2_d128<true>" : "flash_fwd_pp2_d128<false>");
+    hipError_t e = fv_internal_launch_flash(&p, causal ? 1 : 0, (int)d, (hipStream_t)stream);
+    if (e != hipSuccess) return fail_hip(e, causal ? "flash_fwd_pp2<causal>" : "flash_fwd_pp2<dense>");
     return FV_OK;
 }
 
@@ -102,7 +102,7 @@ const char* fv_sdpa_arch(void) { return "gfx950"; }
 int fv_sdpa_supported(size_t b, size_t h, size_t sq, size_t sk, size_t d) {
     if (b != 0 && h > (size_t)65535 / b) return 0;
     const size_t bh = b * h;
-    return d == 128 && sq > 0 && sk > 0 && bh >= 1 && bh <= 65535 && sq <= (size_t)INT_MAX &&
+    return (d == 128 || d == 64) && sq > 0 && sk > 0 && bh >= 1 && bh <= 65535 && sq <= (size_t)INT_MAX &&
            sk <= (size_t)INT_MAX;
 }
 

@@ -39,7 +39,7 @@ struct VsaFineParams {
 }  // namespace fv
 
 extern "C" int fv_internal_flash_block_m(void);   // queries per workgroup of the flash kernel in use
-extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal,
+extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal, int d,
                                                hipStream_t stream);
 extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16, const int* slot_src,
                                                    const int* block_sizes, float* out, size_t bh,

@@ -33,13 +33,12 @@ const char* fv_sdpa_last_error(void);
 const char* fv_sdpa_arch(void);
 
 /* rt/attn.rs:112-128 `mma_sdpa_supported`: 1 when the fused kernel takes a
- * [b,h,sq,d] x [b,h,sk,d] call: d == 128, sq > 0, sk > 0, 1 <= b*h <= 65535,
- * lengths fit int32. (The reference's d == 64 variant serves audio models that
- * are outside this library; such calls decline.) */
+ * [b,h,sq,d] x [b,h,sk,d] call: d == 128 or d == 64, sq > 0, sk > 0,
+ * 1 <= b*h <= 65535, lengths fit int32. */
 int fv_sdpa_supported(size_t b, size_t h, size_t sq, size_t sk, size_t d);
 
 /* rt/attn.rs:283-421 `device_mma_sdpa_with` + kernels/attn2.cu:607-621
- * `flash_mma_fwd2_d128`: out = softmax(scale * q k^T) v.
+ * `flash_mma_fwd2_d128` / `_d64`: out = softmax(scale * q k^T) v.
  * q [bh,sq,128], k/v [bh,sk,128] bf16 bits; out is f32 [bh,sq,128] when
  * out_is_bf16 == 0, else bf16 bits (RNE). scale > 0. */
 int fv_sdpa_dense_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,

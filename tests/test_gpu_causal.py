@@ -1,7 +1,7 @@
 """Parity of the block-causal flash kernel against the oracle (masked composed
 fp32 SDPA and the f64 checker). Cases follow the reference's wan_causal_attn
-table (crates/fastvideo-gpucheck/src/kernels_wan.rs:90-169; its d = 64 rows are
-run at d = 128 here), limit max|delta| <= 1e-2 and cosine >= 0.9999 (the
+table (crates/fastvideo-gpucheck/src/kernels_wan.rs:90-169, every case at d = 128
+and at d = 64), limit max|delta| <= 1e-2 and cosine >= 0.9999 (the
 reference's own limit is 2e-2), plus the schedule invariant of
 kernels_wan.rs:230-261: one block spanning the sequence is bit-identical to the
 dense kernel.
@@ -44,12 +44,13 @@ def fv():
     return fv_sdpa
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("bh,s,bt,win,sink", CASES)
-def test_block_causal_matches_masked_oracle(fv, oracle, bh, s, bt, win, sink):
+def test_block_causal_matches_masked_oracle(fv, oracle, bh, s, bt, win, sink, d):
     import torch
 
-    d, seed = 128, 3000 + s
-    announce(f"causal bh={bh} s={s} block={bt} window={win} sink={sink} seed={seed}")
+    seed = 3000 + s + d
+    announce(f"causal bh={bh} s={s} d={d} block={bt} window={win} sink={sink} seed={seed}")
     q, k, v = qkv(seed, bh, s, s, d)
     mask = oracle.block_causal_dense_mask(bt, win, sink, s, s)
     want = oracle.sdpa_composed(q, k, v, mask=mask)

@@ -1,6 +1,6 @@
 """Parity of the gfx950 dense flash kernel (through the C ABI) against the CPU
 oracle's fp32 composed SDPA. Shapes follow the reference's flash_mma table
-(crates/fastvideo-gpucheck/src/kernels.rs:2286-2297, d = 128 rows) plus the
+(crates/fastvideo-gpucheck/src/kernels.rs:2286-2297, d = 128 and d = 64) plus the
 Wan-shaped benchmark configurations; tolerances: max|delta| <= 1e-2, cosine >= 0.9999 vs the fp32
 oracle on identical bf16-valued inputs, rel_l2 <= 1e-2 vs the oracle on the
 unrounded inputs, <= 2e-3 on rounded inputs (kernels.rs:2314-2328).
@@ -12,7 +12,7 @@ from util import announce, assert_parity, metrics, qkv, randn, sample_rows, to_d
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [  # (bh, sq, sk, std)
+SHAPES = [  # (bh, sq, sk, std) at d = 128
     (1, 1, 1, 1.0),
     (2, 64, 64, 1.0),
     (6, 257, 257, 1.0),
@@ -39,11 +39,16 @@ def fv():
     return fv_sdpa
 
 
-@pytest.mark.parametrize("bh,sq,sk,std", SHAPES)
-def test_dense_matches_composed_oracle(fv, oracle, bh, sq, sk, std):
+# the table's d = 64 rows (kernels.rs:2289, 2292) plus tails and a Wan-sized sequence
+SHAPES_D64 = [(2, 70, 70, 1.0), (4, 1000, 333, 1.0), (1, 1, 1, 1.0), (3, 259, 129, 1.0), (32, 125, 1, 1.0),
+              (2, 2048, 2048, 1.0), (2, 777, 4097, 2.0)]
+
+
+@pytest.mark.parametrize("bh,sq,sk,std,d", [s + (128,) for s in SHAPES] + [s + (64,) for s in SHAPES_D64])
+def test_dense_matches_composed_oracle(fv, oracle, bh, sq, sk, std, d):
     import torch
 
-    d, seed = 128, 1000 + bh * 7 + sq
+    seed = 1000 + bh * 7 + sq + d
     announce(f"dense bh={bh} sq={sq} sk={sk} d={d} std={std} seed={seed}")
     q, k, v = qkv(seed, bh, sq, sk, d, std)
     want = oracle.sdpa_composed(q, k, v)
@@ -62,17 +67,18 @@ def test_dense_matches_composed_oracle(fv, oracle, bh, sq, sk, std):
     assert np.array_equal(got16, oracle.quantize_bf16(got))
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("sk", [1, 2, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 383, 449, 511, 513])
-def test_every_tile_count_parity_and_key_tail(fv, oracle, sk):
+def test_every_tile_count_parity_and_key_tail(fv, oracle, sk, d):
     """The kernel walks the keys two 64-key tiles per phase: odd and even tile counts,
     full and ragged last tiles, one to nine tiles; query tails on both sides of a
     256-query workgroup."""
     import torch
 
-    d, bh = 128, 2
+    bh = 2
     for sq in (1, 259):
-        announce(f"dense tile-count sweep bh={bh} sq={sq} sk={sk}")
-        q, k, v = qkv(5000 + sk, bh, sq, sk, d, 1.0)
+        announce(f"dense tile-count sweep bh={bh} sq={sq} sk={sk} d={d}")
+        q, k, v = qkv(5000 + sk + d, bh, sq, sk, d, 1.0)
         want = oracle.sdpa_composed(q, k, v)
         got = fv.sdpa_dense_bf16(*(to_dev_bf16(x) for x in (q, k, v)), out_bf16=False)
         torch.cuda.synchronize()
@@ -128,13 +134,13 @@ def test_large_scores_exercise_the_rescale(fv, oracle):
 def test_declines(fv):
     import torch
 
-    x = torch.zeros((1, 4, 64), device="cuda", dtype=torch.bfloat16)
+    x = torch.zeros((1, 4, 96), device="cuda", dtype=torch.bfloat16)
     with pytest.raises(fv.FvDeclined):
-        fv.sdpa_dense_bf16(x, x, x)          # d = 64: not built
+        fv.sdpa_dense_bf16(x, x, x)          # d = 96: neither 64 nor 128
     y = torch.zeros((1, 4, 128), device="cuda", dtype=torch.bfloat16)
     with pytest.raises(fv.FvDeclined):
         fv.sdpa_dense_bf16(y, y, y, scale=-1.0)
-    assert fv.sdpa_supported(1, 40, 38001, 38001, 128)
+    assert fv.sdpa_supported(1, 40, 38001, 38001, 128) and fv.sdpa_supported(1, 32, 125, 1, 64)
     assert not fv.sdpa_supported(1, 8, 0, 1024, 128)
     assert not fv.sdpa_supported(2, 40000, 64, 64, 128)
 

@@ -30,10 +30,11 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_supported_table():
-    # rt/attn.rs:932-960, d = 128 rows
+    # rt/attn.rs:932-960
     ok = fv_sdpa.sdpa_supported
     assert ok(1, 40, 38001, 38001, 128) and ok(2, 32, 4097, 1024, 128) and ok(1, 1, 1, 1, 128)
-    for d in (32, 64, 80, 96, 256, 384):
+    assert ok(1, 32, 125, 1, 64)
+    for d in (32, 80, 96, 256, 384):
         assert not ok(1, 8, 1024, 1024, d)
     assert not ok(1, 8, 0, 1024, 128) and not ok(1, 8, 1024, 0, 128)
     assert not ok(0, 8, 1024, 1024, 128) and not ok(2, 40000, 64, 64, 128)
