@@ -8,7 +8,7 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vsa624|vsa512|prep) are for the
+Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep) are for the
 design notes; the driver's line is the default `self`.
 """
 import argparse
@@ -37,7 +37,9 @@ WORKLOADS = {
     "c5cross": (40, 75600, 512, 0, "Wan2.1-14B 720p cross-attention, H=40 Sq=75600 Sk=512"),
     "tiny": (12, 320, 320, 0, "tiny Wan-1.3B-shaped self-attention, H=12 S=320 d=128"),
     "self_d64": (24, 32760, 32760, 0, "head dim 64 self-attention, B=1 H=24 S=32760 d=64 bf16 non-causal"),
+    "vdn32": (12, 49920, 49920, -1, "VDN-H3 window softmax, 32 latent frames x 1560 tokens, chunk 5 radius 1, H=12 d=128"),
 }
+VDN = (0, 1560, 32, 5, 1)   # video_start, frame_tokens, frames, chunk, radius of the vdn32 workload
 
 
 VSA_WORKLOADS = {
@@ -193,6 +195,17 @@ def bench_prep(args):
 def visible_pairs(sq, sk, bt):
     if bt == 0:
         return sq * sk
+    if bt < 0:   # VDN window: frames seen per query frame x frame_tokens^2
+        vs, t, frames, c, r = VDN
+        total = 0
+        for f in range(frames):
+            if f in (0, frames - 1):
+                seen = frames
+            else:
+                lo, hi = max(0, (f // c - r) * c), min(frames - 1, (f // c + r + 1) * c - 1)
+                seen = len(set(range(lo, hi + 1)) | {0, frames - 1})
+            total += seen * t * t
+        return total
     total = 0
     for qb in range((sq + bt - 1) // bt):
         nq = min(bt, sq - qb * bt)
@@ -280,7 +293,10 @@ def main():
     scale = 1.0 / d ** 0.5
 
     def step():
-        if bt:
+        if bt < 0:
+            rc = lib.fv_sdpa_vdn_window_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                             args.out_bf16, h, sq, sk, d, scale, *VDN, stream)
+        elif bt:
             rc = lib.fv_sdpa_block_causal_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                                args.out_bf16, h, sq, sk, d, scale, bt, 0, 0, stream)
         else:
@@ -344,7 +360,7 @@ def main():
                      "min_hbm_bytes": bytes_min,
                      "hbm_frac_at_min_traffic": round(bytes_min / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
     }
-    if args.cpu_seconds > 0:
+    if args.cpu_seconds > 0 and bt >= 0:   # the row-sampled oracle takes dense and block-causal masks
         rec["cpu_baseline"] = cpu_baseline(h, sq, sk, d, bt, flops, q, k, v, args.cpu_seconds)
     print(json.dumps(rec), flush=True)
 

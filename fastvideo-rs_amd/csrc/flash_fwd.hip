@@ -2,7 +2,9 @@
 //
 // Replaces the reference's flash_mma_fwd2_d128 / flash_mma_fwd2_causal_d128
 // (crates/fastvideo-cudarc/src/rt/kernels/attn2.cu:40-352) behind
-// attn::device_mma_sdpa / device_mma_sdpa_causal (rt/attn.rs:225-421, 652-730).
+// attn::device_mma_sdpa / device_mma_sdpa_causal (rt/attn.rs:225-421, 652-730), and
+// flash_mma_fwd2_window_d128 (attn2.cu:356-578) behind device_mma_sdpa_window
+// (rt/attn.rs:526-610).
 //
 // Schedule (not a translation of the CUDA one):
 //   * one workgroup = 8 waves = 256 queries of one (batch, head); each wave
@@ -51,8 +53,9 @@
 // before phase m+1 of either group reads them. V buffers 2 and 3 start as zeros
 // (phase 0 multiplies them with P = 0). An odd tile count is rounded up: the extra
 // tile re-reads the last one and all its scores are masked. Tile indices are walk
-// positions: for block-causal calls the walk is the sink tiles [0, ns) followed
-// by the band [mlo, mhi).
+// positions: a masked call walks up to three ascending tile ranges (block-causal:
+// sink tiles, then the band; VDN window: rows before the video + frame 0, the
+// window frames, the last frame + rows after the video).
 #include "attn_core.h"
 #include "fv_internal.h"
 
@@ -62,7 +65,7 @@ constexpr int kBN = 64;          // keys per tile
 constexpr int kPpBM = 256;      // queries per workgroup
 constexpr int kRing2 = 4;        // K buffers = V buffers: 128 KB of LDS at D = 128, 64 KB at D = 64
 
-template <bool CAUSAL, int D>
+template <bool MASKED, int D>
 __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     using G = TileGeo<D>;
     constexpr int kD = D;
@@ -76,16 +79,18 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     const int h = lane >> 5, c32 = lane & 31;
     // Work order. Dense (equal tiles): workgroup i runs on XCD i % 8, and XCD x takes the
     // contiguous range [x, x+1) * per_xcd of (head, query tile) items, so its CUs stream one
-    // head's K/V through its L2 together. Block-causal (tiles differ in length by up to the
-    // whole band): longest first over the whole launch, tile index major and head minor;
-    // measured 9 % faster than the dense order, whose per-XCD ranges hold unequal work.
+    // head's K/V through its L2 together. Masked (tiles differ in length by up to the whole
+    // sequence): longest first over the whole launch, tile index major and head minor
+    // (block-causal: last tile first; VDN window: the anchor / global tiles at both ends
+    // first); measured 9 % faster than the dense order, whose per-XCD ranges hold unequal work.
     int bh, qt;
-    if constexpr (CAUSAL) {
+    if constexpr (MASKED) {
         const int work = blockIdx.x;
         if (work >= p.total) return;
         const int nbh = p.total / p.nqt;
         bh = work % nbh;
-        qt = p.nqt - 1 - work / nbh;
+        const int r = work / nbh;
+        qt = p.mask_mode == 2 ? ((r & 1) ? (r >> 1) : p.nqt - 1 - (r >> 1)) : p.nqt - 1 - r;
     } else {
         const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
         if (work >= p.total) return;
@@ -110,29 +115,73 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     const uint16_t* Vh = p.v + (size_t)bh * sk * kD;
 
     const int nkt = (sk + kBN - 1) / kBN;
-    int ns = 0, mlo = 0, ne = nkt;           // walk: tiles [0, ns) then [mlo, mlo + ne - ns)
-    int hi_q = 0, lo_q = 0, sink_tok = 0;
-    if constexpr (CAUSAL) {
-        const int ft = p.ft, win = p.win;
-        const int fq_lo = q0 / ft, fq_hi = (q0 + qlen - 1) / ft;
-        const int hi_tok = (int)min((long)sk, (long)(fq_hi + 1) * ft);
-        const int lo_tok = min(hi_tok, win > 0 ? max(0, fq_lo - win + 1) * ft : 0);
-        sink_tok = (int)min((long)sk, (long)p.sink * ft);
-        const int sink_tiles = (sink_tok + kBN - 1) / kBN;
-        mlo = lo_tok / kBN;
-        const int mhi = max((hi_tok + kBN - 1) / kBN, sink_tiles);
-        ns = min(sink_tiles, mlo);
-        ne = ns + (mhi - mlo);
-        const int tq = (q0 + wave * 32 + c32) / ft;
-        hi_q = (int)min((long)0x7fffffff, (long)(tq + 1) * ft);
-        lo_q = win > 0 ? max(0, tq - win + 1) * ft : 0;
+    // The key-tile walk of this query tile: up to three ascending tile ranges [a_i, a_i + n_i),
+    // n0 + n1 + n2 = ne tiles in all. A lane's query sees key x iff
+    //   x < a_hi  ||  x >= c_lo  ||  (w_lo <= x && x < w_hi).
+    int a1 = 0, a2 = 0, n0 = nkt, n1 = 0, ne = nkt;
+    int a_hi = 0, c_lo = 0x7fffffff, w_lo = 0, w_hi = 0;
+    if constexpr (MASKED) {
+        const int qi = q0 + wave * 32 + c32;   // this lane's query (rows past sq are never stored)
+        int b0, b1, b2 = 0;
+        if (p.mask_mode == 1) {
+            // block-causal (rt/attn.rs:449-453): keys of blocks (tq - win, tq], plus the sink blocks
+            const int ft = p.ft, win = p.win;
+            const int fq_lo = q0 / ft, fq_hi = (q0 + qlen - 1) / ft;
+            const int hi_tok = (int)min((long)sk, (long)(fq_hi + 1) * ft);
+            const int lo_tok = min(hi_tok, win > 0 ? max(0, fq_lo - win + 1) * ft : 0);
+            const int sink_tok = (int)min((long)sk, (long)p.sink * ft);
+            b0 = (sink_tok + kBN - 1) / kBN;                       // sink tiles [0, b0)
+            a1 = lo_tok / kBN;                                     // band [a1, b1)
+            b1 = (hi_tok + kBN - 1) / kBN;
+            const int tq = qi / ft;
+            a_hi = sink_tok;
+            w_hi = (int)min((long)0x7fffffff, (long)(tq + 1) * ft);
+            w_lo = win > 0 ? max(0, tq - win + 1) * ft : 0;
+        } else {
+            // VDN window (rt/attn.rs:483-510): rows outside [vs, ve) and the frames 0 and
+            // frames-1 are dense both ways; any other frame sees the frames of its window
+            const int vs = p.vs, ve = p.ve, t = p.ft, last = p.frames - 1, c = p.chunk, r = p.radius;
+            auto lo_frame = [&](int f) { return max(0, c > 0 ? (f / c - r) * c : f - r); };
+            auto hi_frame = [&](int f) { return min(last, c > 0 ? (f / c + r + 1) * c - 1 : f + r); };
+            const bool inner_tile = q0 >= vs + t && q0 + qlen <= ve - t;   // frames 1 .. last-1 only
+            if (inner_tile) {
+                const int fmin = (q0 - vs) / t, fmax = (q0 + qlen - 1 - vs) / t;
+                b0 = (vs + t + kBN - 1) / kBN;                     // rows before the video + frame 0
+                a1 = (vs + lo_frame(fmin) * t) / kBN;              // the window frames of the tile
+                b1 = (vs + (hi_frame(fmax) + 1) * t + kBN - 1) / kBN;
+                a2 = (ve - t) / kBN;                               // last frame + rows after the video
+                b2 = nkt;
+            } else {
+                b0 = nkt;
+                b1 = 0;
+            }
+            const bool inner_q = qi >= vs + t && qi < ve - t;
+            if (inner_q) {
+                const int qf = (qi - vs) / t;
+                a_hi = vs + t;
+                c_lo = ve - t;
+                w_lo = vs + lo_frame(qf) * t;
+                w_hi = vs + (hi_frame(qf) + 1) * t;
+            } else {
+                a_hi = 0x7fffffff;
+            }
+        }
+        // ranges may touch or overlap: each starts no earlier than the previous one ends
+        b0 = min(b0, nkt);
+        a1 = max(a1, b0);
+        b1 = min(max(b1, a1), nkt);
+        a2 = max(a2, b1);
+        b2 = max(b2, a2);
+        n0 = b0;
+        n1 = b1 - a1;
+        ne = n0 + n1 + (min(b2, nkt) - min(a2, nkt));
     }
-    if (ne <= 0) return;   // cannot happen for sk >= 1 (the walk always holds the query's own block)
+    if (ne <= 0) return;   // cannot happen for sk >= 1 (a walk always holds the query's own keys)
     const int np = (ne + 1) / 2;             // phases
     // first key of walk position e; positions past the end repeat the last tile (their scores are masked)
     auto kv0_of = [&](int e) -> int {
         e = min(e, ne - 1);
-        if constexpr (CAUSAL) return (e < ns ? e : mlo + (e - ns)) * kBN;
+        if constexpr (MASKED) return (e < n0 ? e : e < n0 + n1 ? a1 + (e - n0) : a2 + (e - n0 - n1)) * kBN;
         else return e * kBN;
     };
     // tile t lives in buffer t mod 4 (t >= -2)
@@ -199,7 +248,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     if (grp == 1) block_barrier();   // group 1 idles through slot 0
 
     // scores of walk position e: keys past the end (or a position past the walk) to -inf;
-    // block-causal: keys this lane's query may not see to -inf, skipped when the whole
+    // masked launches: keys this lane's query may not see to -inf, skipped when the whole
     // wave sees the whole tile
     auto mask_tile = [&](f32x16 (&s)[2], int e) {
         const int kv0 = kv0_of(e);
@@ -213,16 +262,16 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                     if (key >= lim) s[b][i] = NEG;
                 }
         }
-        if constexpr (CAUSAL) {
+        if constexpr (MASKED) {
             const int kend = min(kv0 + kBN, sk);
-            const bool lane_all = (kend <= hi_q && kv0 >= lo_q) || kend <= sink_tok;
+            const bool lane_all = kend <= a_hi || kv0 >= c_lo || (kv0 >= w_lo && kend <= w_hi);
             if (__builtin_amdgcn_ballot_w64(!lane_all) != 0) {
 #pragma unroll
                 for (int b = 0; b < 2; b++)
 #pragma unroll
                     for (int i = 0; i < 16; i++) {
                         const int key = kv0 + 32 * b + 8 * (i >> 2) + 4 * h + (i & 3);
-                        const bool vis = (key < hi_q && key >= lo_q) || key < sink_tok;
+                        const bool vis = key < a_hi || key >= c_lo || (key >= w_lo && key < w_hi);
                         if (!vis) s[b][i] = NEG;
                     }
             }
@@ -233,7 +282,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     for (int m = 0; m < np; m++) {
         // ---- matrix phase: group 0 in slot 2m, group 1 in slot 2m+1 ----
         __builtin_amdgcn_s_setprio(1);
-        constexpr int kAhead = CAUSAL ? 2 : 3;
+        constexpr int kAhead = MASKED ? 2 : 3;
         // DMA issue slots: after groups 1, 2 (first tile of the pair) and 4, 5 (second) at
         // D = 128; after groups 1 and 3 at D = 64 (one instruction per tile and wave)
         auto hook_k = [&](int g) {
@@ -317,20 +366,20 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
 extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 
 namespace {
-template <bool CAUSAL, int D>
+template <bool MASKED, int D>
 hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
     static std::atomic<unsigned long long> attr_done;
     constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
-    hipError_t e = fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<CAUSAL, D>, lds, attr_done);
+    hipError_t e = fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<MASKED, D>, lds, attr_done);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((fv::flash_fwd_pp2<CAUSAL, D>), dim3(p->per_xcd * 8), dim3(512), lds, stream, *p);
+    hipLaunchKernelGGL((fv::flash_fwd_pp2<MASKED, D>), dim3(p->per_xcd * 8), dim3(512), lds, stream, *p);
     return hipGetLastError();
 }
 }  // namespace
 
-extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal, int d,
+extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int masked, int d,
                                                hipStream_t stream) {
-    if (d == 128) return causal ? launch_flash<true, 128>(p, stream) : launch_flash<false, 128>(p, stream);
-    if (d == 64) return causal ? launch_flash<true, 64>(p, stream) : launch_flash<false, 64>(p, stream);
+    if (d == 128) return masked ? launch_flash<true, 128>(p, stream) : launch_flash<false, 128>(p, stream);
+    if (d == 64) return masked ? launch_flash<true, 64>(p, stream) : launch_flash<false, 64>(p, stream);
     return hipErrorInvalidValue;
 }

@@ -51,9 +51,17 @@ __global__ void cast_bf16_f32_kernel(const uint16_t* __restrict__ x, float* __re
     if (i < n) y[i] = fv::bf16_bits_to_f32(x[i]);
 }
 
+enum { kMaskNone = 0, kMaskBlockCausal = 1, kMaskVdnWindow = 2 };
+
+struct MaskArgs {
+    int mode = kMaskNone;
+    size_t block_tokens = 0, window = 0, sink = 0;                           // block-causal
+    size_t video_start = 0, frame_tokens = 0, frames = 0, chunk = 0, radius = 0;   // VDN window
+};
+
 int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                  int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
-                 bool causal, size_t block_tokens, size_t window, size_t sink, void* stream) {
+                 const MaskArgs& m, void* stream) {
     if (!fv_sdpa_supported(1, bh, sq, sk, d)) return decline("sdpa: shape not taken by the fused kernel");
     if (!(scale > 0.0f) || !(scale < 3.0e38f)) return decline("sdpa: the fused kernel needs a finite scale > 0");
     if (!q || !k || !v || !out) return fv_invalid("sdpa: null operand");
@@ -73,22 +81,40 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
     if (total > (size_t)INT_MAX / 2) return decline("sdpa: too many query tiles for one launch");
     p.total = (int)total;
     p.per_xcd = (int)((total + 7) / 8);
+    p.mask_mode = kMaskNone;
     p.ft = p.win = p.sink = 0;
-    if (causal) {
+    p.vs = p.ve = p.frames = p.chunk = p.radius = 0;
+    int mode = m.mode;
+    const size_t lim = (size_t)INT_MAX;
+    if (mode == kMaskBlockCausal) {
         // rt/attn.rs:668-676
-        const size_t lim = (size_t)INT_MAX;
-        if (block_tokens == 0 || window > lim || sink > lim || (sq > sk ? sq : sk) + block_tokens > lim)
+        if (m.block_tokens == 0 || m.window > lim || m.sink > lim || (sq > sk ? sq : sk) + m.block_tokens > lim)
             return decline("sdpa: block-causal parameters outside the kernel's int range");
-        p.ft = (int)block_tokens;
-        p.win = (int)window;
-        p.sink = (int)sink;
+        p.ft = (int)m.block_tokens;
+        p.win = (int)m.window;
+        p.sink = (int)m.sink;
         // One block spanning both sequences: every key is visible to every query (tq == tk == 0
-        // for any window), so this is the dense problem and runs on the dense kernel, bit for bit
+        // for any window), so this is the dense problem and runs as the dense launch, bit for bit
         // (the reference asserts that identity for its own kernels, gpucheck kernels_wan.rs:230-261).
-        if (block_tokens >= sq && block_tokens >= sk) causal = false;
+        if (m.block_tokens >= sq && m.block_tokens >= sk) mode = kMaskNone;
+    } else if (mode == kMaskVdnWindow) {
+        // rt/attn.rs:544-553: self-attention only, the video rows inside the sequence
+        const size_t ve = m.video_start + m.frames * m.frame_tokens;
+        if (sq != sk || m.frames == 0 || m.frame_tokens == 0 || m.frames > lim / m.frame_tokens || ve > sk ||
+            m.chunk > lim || m.radius > lim / 2 || (m.chunk > 0 && m.radius > lim / (2 * m.chunk)))
+            return decline("sdpa: VDN window parameters the kernel cannot run");
+        p.ft = (int)m.frame_tokens;
+        p.vs = (int)m.video_start;
+        p.ve = (int)ve;
+        p.frames = (int)m.frames;
+        p.chunk = (int)m.chunk;
+        // a radius past the clip means every frame: clamp so that (f/c + r + 1) * c stays in int range
+        p.radius = (int)(m.radius > m.frames ? m.frames : m.radius);
+        if (m.frames <= 2) mode = kMaskNone;   // anchors only: dense
     }
-    hipError_t e = fv_internal_launch_flash(&p, causal ? 1 : 0, (int)d, (hipStream_t)stream);
-    if (e != hipSuccess) return fail_hip(e, causal ? "flash_fwd_pp2<causal>" : "flash_fwd_pp2<dense>");
+    p.mask_mode = mode;
+    hipError_t e = fv_internal_launch_flash(&p, mode != kMaskNone ? 1 : 0, (int)d, (hipStream_t)stream);
+    if (e != hipSuccess) return fail_hip(e, mode != kMaskNone ? "flash_fwd_pp2<masked>" : "flash_fwd_pp2<dense>");
     return FV_OK;
 }
 
@@ -109,15 +135,33 @@ int fv_sdpa_supported(size_t b, size_t h, size_t sq, size_t sk, size_t d) {
 int fv_sdpa_dense_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                        int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                        void* stream) {
-    return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, false, 0, 0, 0, stream);
+    return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, MaskArgs{}, stream);
 }
 
 int fv_sdpa_block_causal_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                               int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d,
                               float scale, size_t block_tokens, size_t window, size_t sink,
                               void* stream) {
-    return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, true, block_tokens, window,
-                        sink, stream);
+    MaskArgs m;
+    m.mode = kMaskBlockCausal;
+    m.block_tokens = block_tokens;
+    m.window = window;
+    m.sink = sink;
+    return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, m, stream);
+}
+
+int fv_sdpa_vdn_window_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
+                            int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
+                            size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                            size_t radius, void* stream) {
+    MaskArgs m;
+    m.mode = kMaskVdnWindow;
+    m.video_start = video_start;
+    m.frame_tokens = frame_tokens;
+    m.frames = frames;
+    m.chunk = chunk;
+    m.radius = radius;
+    return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, m, stream);
 }
 
 int fv_cast_f32_bf16(const float* x, uint16_t* y, size_t n, void* stream) {

@@ -102,6 +102,27 @@ void fv_block_causal_dense_mask(size_t block_tokens, size_t window, size_t sink,
             mask[q * sk + k] = fv_block_causal_allows(block_tokens, window, sink, q, k) ? 0.0f : -1e9f;
 }
 
+int fv_vdn_window_allows(size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                         size_t radius, size_t q, size_t k) {
+    const size_t vs = video_start, ve = video_start + frames * frame_tokens, t = frame_tokens ? frame_tokens : 1;
+    if (q < vs || q >= ve || k < vs || k >= ve) return 1;
+    const size_t last = frames - 1;
+    const size_t qf = (q - vs) / t, kf = (k - vs) / t;
+    if (qf == 0 || kf == 0 || qf == last || kf == last) return 1;
+    const long long f = (long long)qf, c = (long long)chunk, r = (long long)radius, kk = (long long)kf;
+    const long long lo = c > 0 ? (f / c - r) * c : f - r;
+    const long long hi = c > 0 ? (f / c + r + 1) * c - 1 : f + r;
+    return kk >= lo && kk <= hi;
+}
+
+void fv_vdn_window_dense_mask(size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                              size_t radius, size_t sq, size_t sk, float* mask) {
+    for (size_t q = 0; q < sq; q++)
+        for (size_t k = 0; k < sk; k++)
+            mask[q * sk + k] =
+                fv_vdn_window_allows(video_start, frame_tokens, frames, chunk, radius, q, k) ? 0.0f : -1e9f;
+}
+
 int fv_block_causal_for(size_t num_frames_per_block, long long local_attn_size, size_t frame_tokens,
                         size_t out3[3]) {
     const size_t fpb = num_frames_per_block ? num_frames_per_block : 1;

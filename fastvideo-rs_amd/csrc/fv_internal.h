@@ -20,7 +20,9 @@ struct FlashParams {
     int nqt;            // query tiles per (batch, head)
     int total;          // bh * nqt
     int per_xcd;        // ceil(total / 8)
-    int ft, win, sink;  // block-causal: block tokens, window blocks, sink blocks
+    int mask_mode;      // 0 none, 1 block-causal, 2 VDN window
+    int ft, win, sink;  // block-causal: block tokens, window blocks, sink blocks; VDN window: ft = frame tokens
+    int vs, ve, frames, chunk, radius;   // VDN window: video rows [vs, ve), frame count, chunk, radius
 };
 
 struct VsaFineParams {
@@ -39,7 +41,7 @@ struct VsaFineParams {
 }  // namespace fv
 
 extern "C" int fv_internal_flash_block_m(void);   // queries per workgroup of the flash kernel in use
-extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int causal, int d,
+extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int masked, int d,
                                                hipStream_t stream);
 extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16, const int* slot_src,
                                                    const int* block_sizes, float* out, size_t bh,

@@ -172,10 +172,11 @@ float default_scale(std::optional<float> scale, size_t d) {
     return scale ? *scale : 1.0f / sqrtf((float)d);
 }
 
-// One fused launch (dense or block-causal); nullopt = the kernel declined.
+// One fused launch (dense, block-causal or VDN window); nullopt = the kernel declined.
 Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tensor& v,
                                     std::optional<float> scale, bool out_bf16,
-                                    const BlockCausal* causal, hipStream_t st) {
+                                    const BlockCausal* causal, hipStream_t st,
+                                    const VdnWindow* window = nullptr) {
     const auto s = bhsd(q, k, v);
     if (!s || !fv_sdpa_supported(s->b, s->h, s->sq, s->sk, s->d)) return std::optional<Tensor>{};
     Tensor tq, tk, tv;
@@ -196,11 +197,15 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
     if (causal)
         rc = fv_sdpa_block_causal_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
                                        causal->block_tokens, causal->window, causal->sink, st);
+    else if (window)
+        rc = fv_sdpa_vdn_window_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
+                                     window->video_start, window->frame_tokens, window->frames, window->chunk,
+                                     window->radius, st);
     else
         rc = fv_sdpa_dense_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc, st);
     if (rc == FV_DECLINED) return std::optional<Tensor>{};
     if (rc != FV_OK) return msg("sdpa: " + rc_message(rc));
-    (causal ? g_causal : g_fused)++;
+    ((causal || window) ? g_causal : g_fused)++;
     return std::optional<Tensor>{std::move(out)};
 }
 
@@ -255,6 +260,23 @@ Result<Tensor> block_causal(const Tensor& q, const Tensor& k, const Tensor& v, s
         auto& o = std::get<std::optional<Tensor>>(r);
         if (o) return std::move(*o);
     }
+    auto m = upload_mask(mask.dense_mask(sq, sk), sq, sk, st);
+    if (!is_ok(m)) return m;
+    return dense(q, k, v, scale, &std::get<Tensor>(m), st);
+}
+
+// rt/sdpa.rs:271-298
+Result<Tensor> vdn_window(const Tensor& q, const Tensor& k, const Tensor& v, std::optional<float> scale,
+                          VdnWindow mask, hipStream_t st) {
+    const size_t sq = q.shape[2], sk = k.shape[2];
+    auto r = fused(q, k, v, scale, bf16_activations(), nullptr, st, &mask);
+    if (!is_ok(r)) return std::get<TensorError>(r);
+    auto& o = std::get<std::optional<Tensor>>(r);
+    if (o) return std::move(*o);
+    // The masked fallback materialises [sq, sk]: small (test) shapes only.
+    if (sq != 0 && sk > ((size_t)1 << 26) / sq)
+        return msg("sdpa_vdn_window: the window kernel cannot run this " + std::to_string(sq) + "x" +
+                   std::to_string(sk) + " call and the dense mask is too large");
     auto m = upload_mask(mask.dense_mask(sq, sk), sq, sk, st);
     if (!is_ok(m)) return m;
     return dense(q, k, v, scale, &std::get<Tensor>(m), st);
@@ -342,6 +364,15 @@ bool BlockCausal::allows(size_t q, size_t k) const {
 std::vector<float> BlockCausal::dense_mask(size_t sq, size_t sk) const {
     std::vector<float> m(sq * sk);
     fv_block_causal_dense_mask(block_tokens, window, sink, sq, sk, m.data());
+    return m;
+}
+
+bool VdnWindow::allows(size_t q, size_t k) const {
+    return fv_vdn_window_allows(video_start, frame_tokens, frames, chunk, radius, q, k) != 0;
+}
+std::vector<float> VdnWindow::dense_mask(size_t sq, size_t sk) const {
+    std::vector<float> m(sq * sk);
+    fv_vdn_window_dense_mask(video_start, frame_tokens, frames, chunk, radius, sq, sk, m.data());
     return m;
 }
 
@@ -474,7 +505,7 @@ Result<Tensor> sdpa(const Tensor& q, const Tensor& k, const Tensor& v, const Pla
         case Plan::Kind::BlockCausalK:
             return block_causal(q, k, v, plan.scale, plan.causal, st);
         case Plan::Kind::VdnWindowK:
-            return msg("sdpa_vdn_window: the VDN-H3 window plan is not built for gfx950");
+            return vdn_window(q, k, v, plan.scale, plan.window, st);
         case Plan::Kind::KvWindow:
             return kv_window(q, k, v, plan.kv_flash.value_or(causal_flash_enabled()), st);
     }
@@ -512,7 +543,8 @@ int fv_rt_sdpa(const fv_tensor* q, const fv_tensor* k, const fv_tensor* v, const
             p = Plan::block_causal(scale, BlockCausal{plan->block_tokens, plan->window, plan->sink});
             break;
         case FV_PLAN_VDN_WINDOW:
-            p = Plan::vdn_window(scale, VdnWindow{});
+            p = Plan::vdn_window(scale, VdnWindow{plan->video_start, plan->frame_tokens, plan->frames, plan->chunk,
+                                                  plan->radius});
             break;
         case FV_PLAN_KV_WINDOW:
             p = plan->kv_flash < 0 ? Plan::kv_window() : Plan::kv_window_with(plan->kv_flash != 0);

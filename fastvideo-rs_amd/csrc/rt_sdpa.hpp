@@ -66,10 +66,12 @@ struct BlockCausal {
     std::vector<float> dense_mask(size_t sq, size_t sk) const;
 };
 
-// rt/attn.rs:469-524 — VDN-H3's window mask. Carried so that plans built for it
-// are refused with a message instead of being mis-run; its kernel is not built.
+// rt/attn.rs:469-524 — VDN-H3's window mask.
 struct VdnWindow {
     size_t video_start = 0, frame_tokens = 0, frames = 0, chunk = 0, radius = 0;
+    size_t video_end() const { return video_start + frames * frame_tokens; }
+    bool allows(size_t q, size_t k) const;
+    std::vector<float> dense_mask(size_t sq, size_t sk) const;
 };
 
 // rt/sdpa.rs:29-137

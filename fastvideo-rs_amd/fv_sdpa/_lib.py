@@ -47,6 +47,10 @@ SIGNATURES = {
     "fv_block_causal_dense_mask": (None, [_sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_block_causal_for": (C.c_int, [_sz, C.c_longlong, _sz, _vp]),
     "fv_sp_shard_ranges": (None, [_sz, _sz, _vp]),
+    "fv_sdpa_vdn_window_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float,
+                                          _sz, _sz, _sz, _sz, _sz, _vp]),
+    "fv_vdn_window_allows": (C.c_int, [_sz, _sz, _sz, _sz, _sz, _sz, _sz]),
+    "fv_vdn_window_dense_mask": (None, [_sz, _sz, _sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_qk_norm_rope_bhsd": (C.c_int, [_vp, C.c_int, _vp, C.c_int, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz,
                                        _sz, C.c_float, _vp]),
     "fv_split_heads_bhsd": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz, _sz, _vp]),

@@ -9,7 +9,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["sdpa_dense_bf16", "sdpa_block_causal_bf16", "cast_f32_bf16", "cast_bf16_f32", "sdpa_supported"]
+__all__ = ["sdpa_dense_bf16", "sdpa_block_causal_bf16", "sdpa_vdn_window_bf16", "cast_f32_bf16", "cast_bf16_f32", "sdpa_supported"]
 
 
 def _stream():
@@ -52,6 +52,16 @@ def sdpa_block_causal_bf16(q, k, v, block_tokens, window=0, sink=0, scale=None, 
     _lib.check(_lib.lib().fv_sdpa_block_causal_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                                     int(out_bf16), bh, sq, sk, d, scale, block_tokens, window,
                                                     sink, _stream()))
+    return out
+
+
+def sdpa_vdn_window_bf16(q, k, v, video_start, frame_tokens, frames, chunk=0, radius=0, scale=None, out_bf16=False):
+    bh, sq, sk, d = _bhsd(q, k, v)
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    out = torch.empty((bh, sq, d), device=q.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    _lib.check(_lib.lib().fv_sdpa_vdn_window_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                                  int(out_bf16), bh, sq, sk, d, scale, video_start, frame_tokens,
+                                                  frames, chunk, radius, _stream()))
     return out
 
 

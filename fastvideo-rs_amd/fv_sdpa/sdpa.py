@@ -9,7 +9,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["Plan", "BlockCausal", "sdpa", "with_bf16_act", "bf16_activations", "rt_stats", "TensorError"]
+__all__ = ["Plan", "BlockCausal", "VdnWindow", "sdpa", "with_bf16_act", "bf16_activations", "rt_stats", "TensorError"]
 
 
 class TensorError(RuntimeError):
@@ -23,7 +23,8 @@ class _FvTensor(C.Structure):
 class _FvPlan(C.Structure):
     _fields_ = [("kind", C.c_int), ("has_scale", C.c_int), ("scale", C.c_float), ("mask", C.POINTER(_FvTensor)),
                 ("fp8_first", C.c_int), ("block_tokens", C.c_size_t), ("window", C.c_size_t), ("sink", C.c_size_t),
-                ("kv_flash", C.c_int)]
+                ("video_start", C.c_size_t), ("frame_tokens", C.c_size_t), ("frames", C.c_size_t),
+                ("chunk", C.c_size_t), ("radius", C.c_size_t), ("kv_flash", C.c_int)]
 
 
 class BlockCausal:
@@ -41,13 +42,38 @@ class BlockCausal:
         return block_causal_dense_mask(self.block_tokens, self.window, self.sink, sq, sk)
 
 
+class VdnWindow:
+    """rt/attn.rs:469-524."""
+
+    def __init__(self, video_start, frame_tokens, frames, chunk=0, radius=0):
+        self.video_start, self.frame_tokens, self.frames, self.chunk, self.radius = (video_start, frame_tokens,
+                                                                                     frames, chunk, radius)
+
+    def _args(self):
+        return self.video_start, self.frame_tokens, self.frames, self.chunk, self.radius
+
+    def video_end(self):
+        return self.video_start + self.frames * self.frame_tokens
+
+    def allows(self, q, k):
+        return bool(_lib.lib().fv_vdn_window_allows(*self._args(), q, k))
+
+    def dense_mask(self, sq, sk):
+        import numpy as np
+
+        m = np.empty((sq, sk), dtype=np.float32)
+        _lib.lib().fv_vdn_window_dense_mask(*self._args(), sq, sk, m.ctypes.data)
+        return m
+
+
 class Plan:
     """rt/sdpa.rs:29-137."""
 
     DENSE, COMPOSED, BLOCK_CAUSAL, VDN_WINDOW, KV_WINDOW = range(5)
 
-    def __init__(self, kind, scale=None, mask=None, fp8=False, causal=None, kv_flash=None):
+    def __init__(self, kind, scale=None, mask=None, fp8=False, causal=None, kv_flash=None, window=None):
         self.kind, self.scale, self.mask, self.fp8, self.causal, self.kv_flash = kind, scale, mask, fp8, causal, kv_flash
+        self.window = window
 
     @staticmethod
     def dense(scale=None):
@@ -71,8 +97,8 @@ class Plan:
         return Plan(Plan.BLOCK_CAUSAL, scale, causal=mask)
 
     @staticmethod
-    def vdn_window(scale=None):
-        return Plan(Plan.VDN_WINDOW, scale)
+    def vdn_window(scale, mask):
+        return Plan(Plan.VDN_WINDOW, scale, window=mask)
 
     @staticmethod
     def kv_window():
@@ -124,6 +150,8 @@ def sdpa(q, k, v, plan):
     p.fp8_first = int(plan.fp8)
     if plan.causal is not None:
         p.block_tokens, p.window, p.sink = plan.causal.block_tokens, plan.causal.window, plan.causal.sink
+    if plan.window is not None:
+        p.video_start, p.frame_tokens, p.frames, p.chunk, p.radius = plan.window._args()
     p.kv_flash = -1 if plan.kv_flash is None else int(plan.kv_flash)
     out = _FvTensor()
     stream = torch.cuda.current_stream().cuda_stream

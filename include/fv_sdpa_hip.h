@@ -55,6 +55,17 @@ int fv_sdpa_block_causal_bf16(const uint16_t* q, const uint16_t* k, const uint16
                               float scale, size_t block_tokens, size_t window, size_t sink,
                               void* stream);
 
+/* rt/attn.rs:526-610 `device_mma_sdpa_window` + kernels/attn2.cu:356-578, 648-663
+ * `flash_mma_fwd2_window_d128`: the dense kernel under the VDN-H3 window mask (see
+ * fv_vdn_window_allows): a key-tile walk over at most three ranges per query tile (rows before the
+ * video + frame 0, the window frames of the tile, the last frame + rows after the video), per-score
+ * masking on boundary tiles only. Self-attention (sq == sk), frames > 0, frame_tokens > 0, the video
+ * rows inside the sequence; otherwise declines. */
+int fv_sdpa_vdn_window_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
+                            int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
+                            size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                            size_t radius, void* stream);
+
 /* rt/ops.rs:258-265 `cast_f32_bf16_device` + kernels/core.cu:121: f32 -> bf16
  * bits, RNE, NaN quiet, overflow to inf (kernels/core.cu:6-15). */
 int fv_cast_f32_bf16(const float* x, uint16_t* y, size_t n, void* stream);
@@ -82,7 +93,7 @@ enum {
     FV_PLAN_DENSE = 0,        /* Plan::dense / Plan::masked / .fp8_first() (rt/sdpa.rs:56-88) */
     FV_PLAN_COMPOSED = 1,     /* Plan::composed (rt/sdpa.rs:93-98) */
     FV_PLAN_BLOCK_CAUSAL = 2, /* Plan::block_causal (rt/sdpa.rs:104-109) */
-    FV_PLAN_VDN_WINDOW = 3,   /* Plan::vdn_window (rt/sdpa.rs:114-119): refused, kernel not built */
+    FV_PLAN_VDN_WINDOW = 3,   /* Plan::vdn_window (rt/sdpa.rs:111-119) */
     FV_PLAN_KV_WINDOW = 4     /* Plan::kv_window / kv_window_with (rt/sdpa.rs:125-137) */
 };
 
@@ -93,6 +104,7 @@ typedef struct fv_plan {
     const fv_tensor* mask;    /* additive [.., sq, sk] for DENSE / COMPOSED, else NULL */
     int fp8_first;            /* accepted and ignored: this library is bf16 only */
     size_t block_tokens, window, sink;   /* BLOCK_CAUSAL */
+    size_t video_start, frame_tokens, frames, chunk, radius;   /* VDN_WINDOW (rt/attn.rs:474-481) */
     int kv_flash;             /* KV_WINDOW: -1 = FASTVIDEO_WAN_CAUSAL_FLASH, 0 composed f32, 1 dense route */
 } fv_plan;
 
@@ -200,6 +212,15 @@ int fv_block_causal_allows(size_t block_tokens, size_t window, size_t sink, size
 /* rt/attn.rs:456-466 `BlockCausal::dense_mask`: host [sq, sk], 0 visible / -1e9 masked. */
 void fv_block_causal_dense_mask(size_t block_tokens, size_t window, size_t sink, size_t sq,
                                 size_t sk, float* mask);
+/* rt/attn.rs:497-510 `VdnWindow::allows`: rows outside [video_start, video_start +
+ * frames*frame_tokens) and the frames 0 and frames-1 are dense both ways; any other video query
+ * frame sees the key frames of its window (chunk-aligned, radius chunks each side; chunk == 0 is a
+ * centred frame window). */
+int fv_vdn_window_allows(size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                         size_t radius, size_t q, size_t k);
+/* rt/attn.rs:513-523 `VdnWindow::dense_mask`: host [sq, sk], 0 visible / -1e9 masked. */
+void fv_vdn_window_dense_mask(size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                              size_t radius, size_t sq, size_t sk, float* mask);
 /* rt/attn.rs:630-645 `block_causal_for`: 1 and out3 = {block_tokens, window, 0}, or 0 when the
  * token window does not cover whole blocks. */
 int fv_block_causal_for(size_t num_frames_per_block, long long local_attn_size, size_t frame_tokens,

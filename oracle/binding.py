@@ -79,6 +79,9 @@ def _declare(l):
     l.fvo_vsa_tile_mean.argtypes = [_f32p, _i32p, _u32p, _f32p, _sz, _sz, _sz, _sz, C.c_int]
     l.fvo_vsa_coarse_scores.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, C.c_float]
     l.fvo_shard_ranges.argtypes = [_sz, _sz, _szp]
+    l.fvo_vdn_window_allows.argtypes = [_sz, _sz, _sz, _sz, _sz, _sz, _sz]
+    l.fvo_vdn_window_allows.restype = C.c_int
+    l.fvo_vdn_window_dense_mask.argtypes = [_sz, _sz, _sz, _sz, _sz, _sz, _sz, _f32p]
     for fn in (l.fvo_qk_norm_rope_bhsd, l.fvo_wan_qk_norm_rope16):
         fn.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _sz, _sz, _sz, _sz, _sz, _sz, C.c_float]
     l.fvo_split_heads_bhsd.argtypes = [_f32p, _f32p, _sz, _sz, _sz, _sz, _sz, _sz]
@@ -364,3 +367,15 @@ def merge_heads(x):
     out = np.empty((batch, seq, heads * d), dtype=np.float32)
     lib().fvo_merge_heads(_p(x, _f32p), _p(out, _f32p), batch, heads, seq, d)
     return out
+
+
+# ---- VDN-H3 window mask ------------------------------------------------------------------
+
+def vdn_window_allows(video_start, frame_tokens, frames, chunk, radius, q, k):
+    return bool(lib().fvo_vdn_window_allows(video_start, frame_tokens, frames, chunk, radius, q, k))
+
+
+def vdn_window_dense_mask(video_start, frame_tokens, frames, chunk, radius, sq, sk):
+    m = np.empty((sq, sk), dtype=np.float32)
+    lib().fvo_vdn_window_dense_mask(video_start, frame_tokens, frames, chunk, radius, sq, sk, _p(m, _f32p))
+    return m

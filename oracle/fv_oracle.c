@@ -639,3 +639,34 @@ void fvo_merge_heads(const float* src, float* out, size_t batch, size_t heads, s
                 memcpy(out + (b * seq + s) * hd + h * d, src + ((b * heads + h) * seq + s) * d,
                        d * sizeof(float));
 }
+
+/* ---- VDN-H3 window mask --------------------------------------------------------------- */
+
+/* C/rt/attn.rs:487-495 `bound` */
+static long long vdn_bound(long long f, long long c, long long r, int hi) {
+    if (c > 0) return hi ? (f / c + r + 1) * c - 1 : (f / c - r) * c;
+    return hi ? f + r : f - r;
+}
+
+/* C/rt/attn.rs:497-510 */
+int fvo_vdn_window_allows(size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                          size_t radius, size_t q, size_t k) {
+    const size_t vs = video_start, ve = video_start + frames * frame_tokens;
+    const size_t t = frame_tokens > 1 ? frame_tokens : 1;
+    if (!(q >= vs && q < ve) || !(k >= vs && k < ve)) return 1;
+    const size_t last = frames - 1;
+    const size_t qf = (q - vs) / t, kf = (k - vs) / t;
+    if (qf == 0 || kf == 0 || qf == last || kf == last) return 1;
+    const long long kk = (long long)kf;
+    return kk >= vdn_bound((long long)qf, (long long)chunk, (long long)radius, 0) &&
+           kk <= vdn_bound((long long)qf, (long long)chunk, (long long)radius, 1);
+}
+
+/* C/rt/attn.rs:513-523 */
+void fvo_vdn_window_dense_mask(size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                               size_t radius, size_t sq, size_t sk, float* mask) {
+    for (size_t q = 0; q < sq; q++)
+        for (size_t k = 0; k < sk; k++)
+            mask[q * sk + k] =
+                fvo_vdn_window_allows(video_start, frame_tokens, frames, chunk, radius, q, k) ? 0.0f : -1e9f;
+}

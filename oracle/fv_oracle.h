@@ -16,6 +16,10 @@
  *                         == full bit for bit
  *   fvo_sdpa_f64          vs torch float64 softmax(QK^T)V, brute force
  *   fvo_block_causal_*    known answers C/rt/attn.rs:883-930, M/wan/family.rs:146-191
+ *   fvo_vdn_window_*      hand-counted visible sets for the reference's two window forms
+ *                         (chunk 5 / radius 1: 10-15 frames, docs/ports/vdn-h3.md:103-105; the
+ *                         centred window of G/kernels.rs:2860-2868), anchors and global rows
+ *                         dense both ways, symmetry of the anchor rule, brute-force frame maths
  *   fvo_tile_plan/topk_for known answers C/rt/vsa.rs:480-530
  *   fvo_vsa_attention_host all-tiles + zero gate == dense (2e-5), gate tests,
  *                         C/rt/vsa.rs:534-696
@@ -85,6 +89,11 @@ void fvo_block_causal_dense_mask(size_t block_tokens, size_t window, size_t sink
 /* C/rt/attn.rs:630-645; returns 1 and fills out[3] = {block_tokens, window, sink}, or 0 */
 int fvo_block_causal_for(size_t num_frames_per_block, int64_t local_attn_size,
                          size_t frame_tokens, size_t* out3);
+/* C/rt/attn.rs:483-523 — VDN-H3 window mask */
+int fvo_vdn_window_allows(size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                          size_t radius, size_t q, size_t k);
+void fvo_vdn_window_dense_mask(size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
+                               size_t radius, size_t sq, size_t sk, float* mask);
 /* M/wan/family.rs:80-111 */
 void fvo_causal_temporal_mask(const size_t patch[3], size_t num_frames_per_block,
                               int64_t local_attn_size, size_t frames, size_t height,

@@ -63,10 +63,18 @@ def test_non_bhsd_operands_are_refused(fv):
         fv.sdpa(q, q, q, fv.Plan.dense(None))
 
 
-def test_vdn_window_is_refused_not_misrun(fv):
-    q = dev(np.zeros((1, 1, 4, 128), np.float32))
-    with pytest.raises(fv.TensorError, match="vdn_window"):
-        fv.sdpa(q, q, q, fv.Plan.vdn_window(None))
+def test_vdn_window_of_no_frames_is_dense(fv, oracle):
+    """A window without video rows masks nothing (rt/attn.rs:497-501): the kernel declines it
+    (frames == 0) and the masked fallback runs with an all-visible mask."""
+    import torch
+
+    q, k, v = qkv(73, 2, 40, 40, 128)
+    qd, kd, vd = (dev(x.reshape(1, 2, 40, 128)) for x in (q, k, v))
+    with fv.with_bf16_act(False):
+        out = fv.sdpa(qd, kd, vd, fv.Plan.vdn_window(None, fv.VdnWindow(5, 0, 0)))
+    torch.cuda.synchronize()
+    want = oracle.sdpa_composed(q, k, v)
+    assert np.abs(out.cpu().numpy().reshape(2, 40, 128) - want).max() <= 1e-5
 
 
 def test_block_causal_fallback_matches_the_masked_composed_sdpa(fv, oracle):
