@@ -17,7 +17,7 @@ bool fits_int(size_t x) { return x <= (size_t)INT_MAX; }
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct VsaWorkspace {
-    size_t qc, kc, vc, scores, coarse, selected, qt, kt, vt, sparse, total;
+    size_t qc, kc, vc, scores, coarse, selected, qt, kt, vt, total;
 };
 
 VsaWorkspace vsa_layout(size_t bh, size_t nb, size_t topk, size_t dim) {
@@ -38,7 +38,6 @@ VsaWorkspace vsa_layout(size_t bh, size_t nb, size_t topk, size_t dim) {
     w.qt = take(bh * padded * dim * 2);
     w.kt = take(bh * padded * dim * 2);
     w.vt = take(bh * padded * dim * 2);
-    w.sparse = take(bh * padded * dim * 4);
     w.total = off;
     return w;
 }
@@ -217,6 +216,12 @@ int fv_vsa_fine(const uint16_t* qt, const uint16_t* kt, const uint16_t* vt, cons
     p.q_tiles = (int)q_tiles;
     p.total = (int)(bh * q_tiles);
     p.per_xcd = (p.total + 7) / 8;
+    p.final_out = nullptr;
+    p.coarse = nullptr;
+    p.gate = nullptr;
+    p.gate_is_bf16 = 0;
+    p.slot_src = nullptr;
+    p.seq = 0;
     hipError_t e = fv_internal_launch_fine(&p, (hipStream_t)stream);
     return e == hipSuccess ? FV_OK : fv_fail_hip(e, "vsa_fine");
 }
@@ -260,7 +265,6 @@ int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf1
     uint16_t* qt = (uint16_t*)(ws + w.qt);
     uint16_t* kt = (uint16_t*)(ws + w.kt);
     uint16_t* vt = (uint16_t*)(ws + w.vt);
-    float* sparse = (float*)(ws + w.sparse);
     const size_t padded = num_tiles * kTile;
     int rc;
     // 1. tile means (rt/vsa.rs:378-384)
@@ -275,10 +279,32 @@ int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf1
     if ((rc = fv_vsa_tile_qkv(q, qkv_is_bf16, slot_src, qt, bh, seq, padded, dim, stream))) return rc;
     if ((rc = fv_vsa_tile_qkv(k, qkv_is_bf16, slot_src, kt, bh, seq, padded, dim, stream))) return rc;
     if ((rc = fv_vsa_tile_qkv(v, qkv_is_bf16, slot_src, vt, bh, seq, padded, dim, stream))) return rc;
-    if ((rc = fv_vsa_fine(qt, kt, vt, sel, block_sizes, sparse, bh, num_tiles, topk, dim, scale, 0, num_tiles, stream))) return rc;
-    // 5. out = coarse * gate + sparse, back in token order
-    return fv_vsa_combine(sparse, coarse, gate, gate_is_bf16, slot_src, out, bh, seq, dim, num_tiles, 0,
-                          num_tiles, stream);
+    // 5. out = coarse * gate + sparse, back in token order: fused into the fine kernel's epilogue
+    //    (no f32 sparse buffer: 2 x 200 MB of traffic and 200 MB of workspace less at Wan 480p)
+    if (!(scale > 0.0f) || !(scale < 3.0e38f) || !fits_int(padded) || bh * num_tiles > (size_t)INT_MAX / 2)
+        return fv_decline("vsa_attention: needs a finite scale > 0 and a tile count that fits one launch");
+    fv::VsaFineParams p;
+    p.qt = qt;
+    p.kt = kt;
+    p.vt = vt;
+    p.selected = sel;
+    p.block_sizes = block_sizes;
+    p.out = nullptr;
+    p.num_tiles = (int)num_tiles;
+    p.topk = (int)topk;
+    p.sl2 = scale * 1.4426950408889634f;
+    p.q_base = 0;
+    p.q_tiles = (int)num_tiles;
+    p.total = (int)(bh * num_tiles);
+    p.per_xcd = (p.total + 7) / 8;
+    p.final_out = out;
+    p.coarse = coarse;
+    p.gate = gate;
+    p.gate_is_bf16 = gate_is_bf16;
+    p.slot_src = slot_src;
+    p.seq = (long)seq;
+    hipError_t e = fv_internal_launch_fine(&p, (hipStream_t)stream);
+    return e == hipSuccess ? FV_OK : fv_fail_hip(e, "vsa_fine (fused combine)");
 }
 
 }  // extern "C"

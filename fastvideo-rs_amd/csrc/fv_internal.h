@@ -36,6 +36,14 @@ struct VsaFineParams {
     float sl2;
     int q_base, q_tiles;          // query tiles [q_base, q_base + q_tiles)
     int total, per_xcd;           // bh * q_tiles, ceil(total / 8)
+    // Fused combine (whole-op entry): when `final_out` is set the kernel writes
+    // final_out[token] = coarse[tile] * gate[token] + sparse instead of `out`, in token order.
+    float* final_out;             // [bh, seq, 128] f32 or null
+    const float* coarse;          // [bh, num_tiles, 128]
+    const void* gate;             // [bh, seq, 128] f32 / bf16 or null (gate of one)
+    int gate_is_bf16;
+    const int* slot_src;          // [num_tiles * 64]
+    long seq;
 };
 
 }  // namespace fv

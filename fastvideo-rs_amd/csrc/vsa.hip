@@ -414,6 +414,42 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
 
     const float l_tot = pair_sum(st.l_acc);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (p.final_out) {
+        // fused combine (kernels/core.cu:803-835): out[token] = coarse[tile] * gate[token] + sparse,
+        // the product rounded to f32 before the add as on the host; padding slots write nothing
+#pragma clang fp contract(off)
+        const int token = p.slot_src[(size_t)qtile * kTileElems + wave * 32 + c32];
+        if (token < 0) return;
+        const float* co = p.coarse + ((size_t)bh * nb + qtile) * 128;
+        const size_t row = ((size_t)bh * p.seq + token) * 128;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d0 = 32 * db + 8 * g + 4 * h;
+                const f32x4 c4 = *reinterpret_cast<const f32x4*>(co + d0);
+                f32x4 ga = {1.f, 1.f, 1.f, 1.f};
+                if (p.gate) {
+                    if (p.gate_is_bf16) {
+                        const u32x2 raw = *reinterpret_cast<const u32x2*>((const uint16_t*)p.gate + row + d0);
+                        ga[0] = __builtin_bit_cast(float, raw[0] << 16);
+                        ga[1] = __builtin_bit_cast(float, raw[0] & 0xffff0000u);
+                        ga[2] = __builtin_bit_cast(float, raw[1] << 16);
+                        ga[3] = __builtin_bit_cast(float, raw[1] & 0xffff0000u);
+                    } else {
+                        ga = *reinterpret_cast<const f32x4*>((const float*)p.gate + row + d0);
+                    }
+                }
+                f32x4 r;
+#pragma unroll
+                for (int x = 0; x < 4; x++) {
+                    const float sp = o[db][4 * g + x] * inv;
+                    r[x] = c4[x] * ga[x] + sp;
+                }
+                *reinterpret_cast<f32x4*>(p.final_out + row + d0) = r;
+            }
+        return;
+    }
     float* ob = p.out + (((size_t)bh * p.q_tiles + (qtile - p.q_base)) * kTileElems + wave * 32 + c32) * 128;
 #pragma unroll
     for (int db = 0; db < 4; db++)
