@@ -174,7 +174,9 @@ int fv_vsa_combine(const float* sparse, const float* coarse, const void* gate, i
                    size_t num_tiles, size_t q_base, size_t q_tiles, void* stream);
 /* rt/vsa.rs:358-424 `vsa_attention_device` with FineKernel::Mma: tile means -> coarse ->
  * top-k -> tile permute -> fine -> combine, all on `stream`, using caller-provided scratch
- * (fv_vsa_workspace_bytes, 256-byte aligned). topk is clamped to [1, num_tiles]. q/k/v (and
+ * (fv_vsa_workspace_bytes, 256-byte aligned). The combine runs in the fine kernel's epilogue
+ * (same f32 arithmetic, mul then add), so no f32 sparse buffer is part of the scratch.
+ * topk is clamped to [1, num_tiles]. q/k/v (and
  * gate) are f32 or bf16 bits in token order; out f32 [bh, seq, 128]. selected_out: NULL or
  * [bh, num_tiles, topk] to receive the block index lists. */
 size_t fv_vsa_workspace_bytes(size_t bh, size_t num_tiles, size_t topk, size_t dim);
