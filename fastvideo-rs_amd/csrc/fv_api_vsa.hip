@@ -226,16 +226,31 @@ int fv_vsa_fine(const uint16_t* qt, const uint16_t* kt, const uint16_t* vt, cons
     return e == hipSuccess ? FV_OK : fv_fail_hip(e, "vsa_fine");
 }
 
-int fv_vsa_combine(const float* sparse, const float* coarse, const void* gate, int gate_is_bf16,
-                   const int32_t* slot_src, float* out, size_t bh, size_t seq, size_t dim,
-                   size_t num_tiles, size_t q_base, size_t q_tiles, void* stream) {
+static int combine_common(const float* sparse, const float* coarse, const void* gate, int gate_is_bf16,
+                          const int32_t* slot_src, float* out, size_t bh, size_t seq, size_t dim,
+                          size_t num_tiles, size_t q_base, size_t q_tiles, int round16, void* stream) {
     if (!sparse || !coarse || !slot_src || !out) return fv_invalid("vsa_combine: null operand");
     if (bh == 0 || q_tiles == 0) return FV_OK;
     if (dim != 128 || bh > 65535 || !fits_int(num_tiles * kTile) || q_base + q_tiles > num_tiles)
         return fv_decline("vsa_combine: needs dim == 128 and bh <= 65535");
     hipError_t e = fv_internal_launch_combine(sparse, coarse, gate, gate_is_bf16, slot_src, out, bh, seq,
-                                              (int)num_tiles, (int)q_base, (int)q_tiles, (hipStream_t)stream);
+                                              (int)num_tiles, (int)q_base, (int)q_tiles, round16,
+                                              (hipStream_t)stream);
     return e == hipSuccess ? FV_OK : fv_fail_hip(e, "vsa_combine");
+}
+
+int fv_vsa_combine(const float* sparse, const float* coarse, const void* gate, int gate_is_bf16,
+                   const int32_t* slot_src, float* out, size_t bh, size_t seq, size_t dim,
+                   size_t num_tiles, size_t q_base, size_t q_tiles, void* stream) {
+    return combine_common(sparse, coarse, gate, gate_is_bf16, slot_src, out, bh, seq, dim, num_tiles, q_base,
+                          q_tiles, 0, stream);
+}
+
+int fv_vsa_combine_round16(const float* sparse, const float* coarse, const void* gate, int gate_is_bf16,
+                           const int32_t* slot_src, float* out, size_t bh, size_t seq, size_t dim,
+                           size_t num_tiles, size_t q_base, size_t q_tiles, void* stream) {
+    return combine_common(sparse, coarse, gate, gate_is_bf16, slot_src, out, bh, seq, dim, num_tiles, q_base,
+                          q_tiles, 1, stream);
 }
 
 size_t fv_vsa_workspace_bytes(size_t bh, size_t num_tiles, size_t topk, size_t dim) {

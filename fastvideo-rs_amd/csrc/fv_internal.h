@@ -68,7 +68,7 @@ extern "C" hipError_t fv_internal_launch_combine(const float* sparse, const floa
                                                  const void* gate, int gate_is_bf16,
                                                  const int* slot_src, float* out, size_t bh,
                                                  size_t seq, int num_tiles, int q_base, int q_tiles,
-                                                 hipStream_t st);
+                                                 int round16, hipStream_t st);
 
 // Error plumbing of the C ABI (defined in fv_api.hip): the message is kept per thread.
 int fv_fail_hip(hipError_t e, const char* what);   // returns -(int)e

@@ -464,7 +464,10 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
 
 // ---- combine (kernels/core.cu:803-835) -----------------------------------------------------
 // out[token] = coarse[tile] * gate[token] + sparse[slot]; gate == null is a gate of one.
-template <bool GATE_BF16>
+// ROUND16 is the bf16 combine of the H3 family (kernels/core.cu:825-830, kernels/attn3.cu:247-270):
+// bf16(bf16(sparse) + bf16(bf16(coarse) * bf16(gate))), every step rounded to nearest even and the
+// result stored as the f32 of that bf16 value; without a gate the product is bf16(coarse) itself.
+template <bool GATE_BF16, bool ROUND16>
 __global__ __launch_bounds__(256) void vsa_combine_kernel(
     const float* __restrict__ sparse, const float* __restrict__ coarse,
     const void* __restrict__ gate, const int* __restrict__ slot_src, float* __restrict__ out,
@@ -495,8 +498,18 @@ __global__ __launch_bounds__(256) void vsa_combine_kernel(
         }
     }
     f32x4 r;
+    if constexpr (ROUND16) {
+        auto r16 = [](float x) { return bf16_bits_to_f32(bf16_rne_bits(x)); };
 #pragma unroll
-    for (int e = 0; e < 4; e++) r[e] = co[e] * ga[e] + sp[e];
+        for (int e = 0; e < 4; e++) {
+            const float c = r16(co[e]);
+            const float p = has_gate ? r16(c * r16(ga[e])) : c;
+            r[e] = r16(r16(sp[e]) + p);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) r[e] = co[e] * ga[e] + sp[e];
+    }
     *reinterpret_cast<f32x4*>(out + (bh * seq + src) * 128 + d0) = r;
 }
 
@@ -566,14 +579,19 @@ extern "C" hipError_t fv_internal_launch_combine(const float* sparse, const floa
                                                  const void* gate, int gate_is_bf16,
                                                  const int* slot_src, float* out, size_t bh,
                                                  size_t seq, int num_tiles, int q_base, int q_tiles,
-                                                 hipStream_t st) {
+                                                 int round16, hipStream_t st) {
     const dim3 grid((unsigned)(((size_t)q_tiles * kTileElems + 7) / 8), (unsigned)bh), block(256);
     const int has_gate = gate != nullptr;
-    if (gate_is_bf16)
-        hipLaunchKernelGGL(vsa_combine_kernel<true>, grid, block, 0, st, sparse, coarse, gate, slot_src, out,
-                           (long)seq, num_tiles, q_base, q_tiles, has_gate);
-    else
-        hipLaunchKernelGGL(vsa_combine_kernel<false>, grid, block, 0, st, sparse, coarse, gate, slot_src, out,
-                           (long)seq, num_tiles, q_base, q_tiles, has_gate);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, block, 0, st, sparse, coarse, gate, slot_src, out, (long)seq, num_tiles,
+                           q_base, q_tiles, has_gate);
+    };
+    if (gate_is_bf16) {
+        if (round16) launch(vsa_combine_kernel<true, true>);
+        else launch(vsa_combine_kernel<true, false>);
+    } else {
+        if (round16) launch(vsa_combine_kernel<false, true>);
+        else launch(vsa_combine_kernel<false, false>);
+    }
     return hipGetLastError();
 }

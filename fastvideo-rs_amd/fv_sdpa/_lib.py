@@ -40,6 +40,7 @@ SIGNATURES = {
     "fv_vsa_tile_qkv": (C.c_int, [_vp, C.c_int, _vp, _vp, _sz, _sz, _sz, _sz, _vp]),
     "fv_vsa_fine": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_float, _sz, _sz, _vp]),
     "fv_vsa_combine": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _vp]),
+    "fv_vsa_combine_round16": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_vsa_workspace_bytes": (_sz, [_sz, _sz, _sz, _sz]),
     "fv_vsa_attention": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp, C.c_int, _vp, _vp, _vp, _vp, _sz, _vp,
                                    _sz, _sz, _sz, _sz, _sz, C.c_float, _vp]),

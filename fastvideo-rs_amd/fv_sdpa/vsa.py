@@ -135,7 +135,9 @@ def vsa_fine(qt, kt, vt, selected, ctx, scale, q_base=0, q_tiles=None):
     return out
 
 
-def vsa_combine(sparse, coarse, gate, ctx, out=None, q_base=0, q_tiles=None):
+def vsa_combine(sparse, coarse, gate, ctx, out=None, q_base=0, q_tiles=None, round16=False):
+    """rt/ops.rs:1574-1601 `vsa_combine_device` / `vsa_combine_round_device` (`round16`: the H3
+    family's bf16 combine, every step rounded to bf16)."""
     _chk(sparse, "sparse", (torch.float32,))
     _chk(coarse, "coarse", (torch.float32,))
     bh, nb, dim = coarse.shape
@@ -146,9 +148,10 @@ def vsa_combine(sparse, coarse, gate, ctx, out=None, q_base=0, q_tiles=None):
     if gate is not None:
         _chk(gate, "gate")
         g16 = _is16(gate)
-    _lib.check(_lib.lib().fv_vsa_combine(sparse.data_ptr(), coarse.data_ptr(), gate.data_ptr() if gate is not None else None,
-                                         g16, ctx.slot_src.data_ptr(), out.data_ptr(), bh, ctx.seq, dim, nb, q_base,
-                                         q_tiles, _stream()))
+    entry = _lib.lib().fv_vsa_combine_round16 if round16 else _lib.lib().fv_vsa_combine
+    _lib.check(entry(sparse.data_ptr(), coarse.data_ptr(), gate.data_ptr() if gate is not None else None,
+                     g16, ctx.slot_src.data_ptr(), out.data_ptr(), bh, ctx.seq, dim, nb, q_base,
+                     q_tiles, _stream()))
     return out
 
 

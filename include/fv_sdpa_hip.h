@@ -167,11 +167,18 @@ int fv_vsa_fine(const uint16_t* qt, const uint16_t* kt, const uint16_t* vt, cons
                 size_t dim, float scale, size_t q_base, size_t q_tiles, void* stream);
 /* kernels/core.cu:807-835 `vsa_combine` (rt/ops.rs:1592-1601): out[bh, token, :] =
  * coarse[bh, tile, :] * gate[bh, token, :] + sparse[bh, slot, :] for the real tokens of tiles
- * [q_base, q_base + q_tiles); gate NULL = 1; gate f32 or bf16 bits. dim == 128. (The H3-only
- * `round16` variant, kernels/attn3.cu:247-270, is not built.) */
+ * [q_base, q_base + q_tiles); gate NULL = 1; gate f32 or bf16 bits. dim == 128. */
 int fv_vsa_combine(const float* sparse, const float* coarse, const void* gate, int gate_is_bf16,
                    const int32_t* slot_src, float* out, size_t bh, size_t seq, size_t dim,
                    size_t num_tiles, size_t q_base, size_t q_tiles, void* stream);
+/* `vsa_combine` with round16 = 1 (kernels/core.cu:825-830, rt/ops.rs:1574-1601
+ * `vsa_combine_round_device`) and its bf16-gate twin kernels/attn3.cu:247-270 `vsa_combine_g16`:
+ * the H3 family's bf16 combine, out = bf16(bf16(sparse) + bf16(bf16(coarse) * bf16(gate))), without
+ * a gate bf16(bf16(sparse) + bf16(coarse)); out stays f32 storage holding bf16 values. Same
+ * arguments as fv_vsa_combine. */
+int fv_vsa_combine_round16(const float* sparse, const float* coarse, const void* gate, int gate_is_bf16,
+                           const int32_t* slot_src, float* out, size_t bh, size_t seq, size_t dim,
+                           size_t num_tiles, size_t q_base, size_t q_tiles, void* stream);
 /* rt/vsa.rs:358-424 `vsa_attention_device` with FineKernel::Mma: tile means -> coarse ->
  * top-k -> tile permute -> fine -> combine, all on `stream`, using caller-provided scratch
  * (fv_vsa_workspace_bytes, 256-byte aligned). The combine runs in the fine kernel's epilogue

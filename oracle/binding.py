@@ -77,6 +77,7 @@ def _declare(l):
     l.fvo_topk_device_order.argtypes = [_f32p, _u32p, _sz, _sz, _sz]
     l.fvo_topk_host_order.argtypes = [_f32p, _u32p, _sz, _sz, _sz]
     l.fvo_vsa_tile_mean.argtypes = [_f32p, _i32p, _u32p, _f32p, _sz, _sz, _sz, _sz, C.c_int]
+    l.fvo_vsa_combine.argtypes = [_f32p, _f32p, _f32p, _i32p, _f32p, _sz, _sz, _sz, _sz, _sz, _sz, C.c_int]
     l.fvo_vsa_coarse_scores.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, C.c_float]
     l.fvo_shard_ranges.argtypes = [_sz, _sz, _szp]
     l.fvo_vdn_window_allows.argtypes = [_sz, _sz, _sz, _sz, _sz, _sz, _sz]
@@ -308,6 +309,19 @@ def vsa_tile_mean(x, plan, round16=False):
     out = np.empty((bh, plan.num_tiles, dim), dtype=np.float32)
     lib().fvo_vsa_tile_mean(_p(x, _f32p), _p(plan.slot_src, _i32p), _p(plan.block_sizes, _u32p),
                             _p(out, _f32p), bh, seq, dim, plan.num_tiles, int(round16))
+    return out
+
+
+def vsa_combine(sparse, coarse, gate, plan, seq, round16=False, q_base=0, q_tiles=None, out=None):
+    """C/rt/kernels/core.cu:803-835. sparse [bh, q_tiles*64, dim] tile-slot order, coarse [bh, nb, dim],
+    gate [bh, seq, dim] or None; rows of `out` no tile covers keep their value (zeros if fresh)."""
+    sparse, coarse = _f32(sparse), _f32(coarse)
+    bh, nb, dim = coarse.shape
+    q_tiles = nb - q_base if q_tiles is None else q_tiles
+    gate = _f32(gate) if gate is not None else None
+    out = np.zeros((bh, seq, dim), dtype=np.float32) if out is None else out
+    lib().fvo_vsa_combine(_p(sparse, _f32p), _p(coarse, _f32p), _p(gate, _f32p) if gate is not None else None,
+                          _p(plan.slot_src, _i32p), _p(out, _f32p), bh, seq, dim, nb, q_base, q_tiles, int(round16))
     return out
 
 

@@ -406,6 +406,37 @@ void fvo_vsa_tile_mean(const float* x, const int32_t* slot_src, const uint32_t* 
         }
 }
 
+/* C/rt/kernels/core.cu:803-835 */
+void fvo_vsa_combine(const float* sparse, const float* coarse, const float* gate, const int32_t* slot_src,
+                     float* out, size_t bh, size_t seq, size_t dim, size_t nb, size_t q_base,
+                     size_t q_tiles, int round16) {
+    for (size_t b = 0; b < bh; b++)
+        for (size_t g = 0; g < q_tiles; g++) {
+            const size_t tile = q_base + g;
+            if (tile >= nb) continue;
+            for (size_t slot = 0; slot < 64; slot++) {
+                const int32_t src = slot_src[tile * 64 + slot];
+                if (src < 0) continue;
+                const float* sp = sparse + ((b * q_tiles + g) * 64 + slot) * dim;
+                const float* co = coarse + (b * nb + tile) * dim;
+                const float* ga = gate ? gate + (b * seq + (size_t)src) * dim : NULL;
+                float* ob = out + (b * seq + (size_t)src) * dim;
+                for (size_t d = 0; d < dim; d++) {
+                    if (round16) {
+                        const float c = fvo_bf16_round(co[d]);
+                        const float prod = ga ? c * fvo_bf16_round(ga[d]) : c;
+                        const float p = ga ? fvo_bf16_round(prod) : c;
+                        const float sum = fvo_bf16_round(sp[d]) + p;
+                        ob[d] = fvo_bf16_round(sum);
+                    } else {
+                        const float prod = co[d] * (ga ? ga[d] : 1.0f);
+                        ob[d] = prod + sp[d];
+                    }
+                }
+            }
+        }
+}
+
 void fvo_vsa_coarse_scores(const float* qc, const float* kc, float* scores, size_t bh, size_t nb,
                            size_t dim, float scale) {
     for (size_t b = 0; b < bh; b++)

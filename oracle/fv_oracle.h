@@ -25,6 +25,9 @@
  *                         C/rt/vsa.rs:534-696
  *   fvo_topk_*            brute-force sort on small n, ties, -0.0, both orders
  *   fvo_vsa_tile_mean     closed form on constant/linear inputs
+ *   fvo_vsa_combine       f32 form vs numpy mul-then-add; round16 form vs torch's own bf16
+ *                         multiply and add on CPU tensors, zero gate == bf16(sparse), padding
+ *                         slots leave `out` untouched
  *   fvo_shard_ranges      known answers C/rt/sp.rs:66-84
  *   fvo_qk_norm_rope_bhsd / fvo_wan_qk_norm_rope16
  *                         the two against each other within 0.03 on the closed-form
@@ -122,6 +125,13 @@ void fvo_topk_host_order(const float* scores, uint32_t* out, size_t rows, size_t
 /* C/rt/kernels/core.cu:550-570 — f32 sequential sum in slot order, then / n. */
 void fvo_vsa_tile_mean(const float* x, const int32_t* slot_src, const uint32_t* block_sizes,
                        float* out, size_t bh, size_t seq, size_t dim, size_t nb, int round16);
+/* C/rt/kernels/core.cu:803-835 (bf16 gate: C/rt/kernels/attn3.cu:247-270) — out[token] =
+ * coarse[tile] * gate[token] + sparse[slot] for the real tokens of tiles [q_base, q_base + q_tiles),
+ * gate NULL = 1. round16: bf16(bf16(sparse) + bf16(bf16(coarse) * bf16(gate))), without a gate
+ * bf16(bf16(sparse) + bf16(coarse)). sparse is [bh, q_tiles*64, dim] in tile-slot order. */
+void fvo_vsa_combine(const float* sparse, const float* coarse, const float* gate, const int32_t* slot_src,
+                     float* out, size_t bh, size_t seq, size_t dim, size_t nb, size_t q_base,
+                     size_t q_tiles, int round16);
 /* C/rt/vsa.rs:385-394 restated with a fixed accumulation order (the reference
  * uses cuBLAS f32, whose order is unspecified): scores[qt,kt] =
  * (sum_d in ascending d of qc*kc, f32, no FMA) * scale. */

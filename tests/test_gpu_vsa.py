@@ -141,6 +141,22 @@ def test_tile_qkv_and_combine_bit_exact(fv, oracle, grid):
     b = fv.vsa_combine(dev(sparse), dev(coarse), dev(g16).to(torch.bfloat16), ctx)
     torch.cuda.synchronize()
     assert torch.equal(a, b)
+    # the H3 family's bf16 combine (round16): f32 gate, bf16 gate (same bits), no gate, a tile range
+    for g in (gate, None):
+        wantr = oracle.vsa_combine(sparse, coarse, g, plan, ctx.seq, round16=True)
+        gotr = fv.vsa_combine(dev(sparse), dev(coarse), dev(g) if g is not None else None, ctx, round16=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(gotr.cpu().numpy(), wantr)
+    gotr16 = fv.vsa_combine(dev(sparse), dev(coarse), dev(g16).to(torch.bfloat16), ctx, round16=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(gotr16.cpu().numpy(), oracle.vsa_combine(sparse, coarse, gate, plan, ctx.seq, round16=True))
+    if nb >= 3:
+        part = fv.vsa_combine(dev(sparse[:, 64:(nb * 64)]), dev(coarse), dev(gate), ctx, q_base=1, q_tiles=nb - 1,
+                              round16=True)
+        torch.cuda.synchronize()
+        wantp = oracle.vsa_combine(sparse[:, 64:(nb * 64)], coarse, gate, plan, ctx.seq, round16=True, q_base=1,
+                                   q_tiles=nb - 1)
+        assert np.array_equal(part.cpu().numpy(), wantp)
 
 
 @pytest.mark.parametrize("grid", GRIDS)

@@ -192,6 +192,48 @@ def test_tile_mean_closed_forms(oracle):
     assert np.array_equal(oracle.vsa_tile_mean(x, p, round16=True), np.ones((1, p.num_tiles, 4), np.float32))
 
 
+def test_combine_forms(oracle):
+    """kernels/core.cu:803-835: f32 form = numpy's multiply then add; the round16 form is torch's
+    own bf16 arithmetic (each bf16 op computes in f32 and rounds once), bf16(bf16(sparse) +
+    bf16(bf16(coarse) * bf16(gate))); padding slots and rows outside the tile range are untouched."""
+    import torch
+
+    p = oracle.TilePlan((3, 5, 7))
+    rng = np.random.default_rng(12)
+    bh, dim, nb = 2, 16, p.num_tiles
+    sparse = rng.standard_normal((bh, p.padded, dim)).astype(np.float32)
+    coarse = rng.standard_normal((bh, nb, dim)).astype(np.float32)
+    gate = rng.standard_normal((bh, p.seq, dim)).astype(np.float32)
+    real = p.slot_src >= 0
+    tok, tile = p.slot_src[real], (np.arange(p.padded) // 64)[real]
+    # f32
+    want = np.zeros((bh, p.seq, dim), np.float32)
+    want[:, tok] = (coarse[:, tile] * gate[:, tok]).astype(np.float32) + sparse[:, real]
+    assert np.array_equal(oracle.vsa_combine(sparse, coarse, gate, p, p.seq), want)
+    want[:, tok] = coarse[:, tile] + sparse[:, real]
+    assert np.array_equal(oracle.vsa_combine(sparse, coarse, None, p, p.seq), want)
+    # round16 against torch bf16 tensors
+    b16 = lambda x: torch.from_numpy(x).to(torch.bfloat16)
+    t = b16(sparse[:, real]) + b16(coarse[:, tile]) * b16(gate[:, tok])
+    want = np.zeros((bh, p.seq, dim), np.float32)
+    want[:, tok] = t.float().numpy()
+    got = oracle.vsa_combine(sparse, coarse, gate, p, p.seq, round16=True)
+    assert np.array_equal(got, want)
+    assert not np.array_equal(got, oracle.vsa_combine(sparse, coarse, gate, p, p.seq))
+    t = b16(sparse[:, real]) + b16(coarse[:, tile])
+    want[:, tok] = t.float().numpy()
+    assert np.array_equal(oracle.vsa_combine(sparse, coarse, None, p, p.seq, round16=True), want)
+    # zero gate: bf16(sparse)
+    z = oracle.vsa_combine(sparse, coarse, np.zeros_like(gate), p, p.seq, round16=True)
+    assert np.array_equal(z[:, tok], oracle.quantize_bf16(sparse[:, real]))
+    # a tile range writes only its tokens
+    out = np.full((bh, p.seq, dim), 7.0, np.float32)
+    oracle.vsa_combine(sparse[:, 64:192], coarse, gate, p, p.seq, q_base=1, q_tiles=2, out=out)
+    inside = np.zeros(p.seq, bool)
+    inside[p.slot_src[64:192][p.slot_src[64:192] >= 0]] = True
+    assert np.all(out[:, ~inside] == 7.0) and np.all(out[:, inside] != 7.0)
+
+
 def test_coarse_scores_vs_f64(oracle):
     rng = np.random.default_rng(3)
     qc = rng.standard_normal((2, 9, 128)).astype(np.float32)
