@@ -2,6 +2,7 @@
 // See rt_sdpa.hpp for the reference citations.
 #include "rt_sdpa.hpp"
 
+#include <ctype.h>
 #include <limits.h>
 #include <math.h>
 #include <stdlib.h>
@@ -110,6 +111,17 @@ TensorError msg(std::string s) { return TensorError{std::move(s)}; }
 
 std::atomic<uint64_t> g_fused{0}, g_causal{0}, g_composed{0}, g_cast{0}, g_masks{0};
 thread_local std::optional<bool> g_bf16_override;
+thread_local std::optional<Backend> g_backend_override;
+
+// rt/sdpa.rs:234-246 `retired`
+std::string retired(Backend b) {
+    if (b == Backend::Sparse)
+        return "FASTVIDEO_SDPA=sparse (the host block-sparse window prototype) is retired: "
+               "FASTVIDEO_VSA=1 selects video sparse attention on the device; unset FASTVIDEO_SDPA for "
+               "dense attention";
+    return "FASTVIDEO_SDPA=host (the host online-softmax attention) is retired: unset FASTVIDEO_SDPA "
+           "for the dense default";
+}
 
 bool env_flag(const char* name, bool dflt) {
     const char* v = getenv(name);
@@ -209,16 +221,23 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
     return std::optional<Tensor>{std::move(out)};
 }
 
-// rt/sdpa.rs:184-214 `dense` with the collapsed route [Mma, Composed] / [Composed].
+// rt/sdpa.rs:184-233 `dense` / `run_step` over the collapsed route.
 Result<Tensor> dense(const Tensor& q, const Tensor& k, const Tensor& v, std::optional<float> scale,
                      const Tensor* mask, hipStream_t st) {
     const bool act16 = bf16_activations();
-    if (!mask) {
-        auto r = fused(q, k, v, scale, act16, nullptr, st);
-        if (!is_ok(r)) return std::get<TensorError>(r);
-        auto& o = std::get<std::optional<Tensor>>(r);
-        if (o) return std::move(*o);
+    const Backend be = backend();
+    bool composed_step = false;
+    for (Step step : dense_route(Shape::of(q.shape, k.shape, v.shape), mask != nullptr, be)) {
+        if (step == Step::Retired) return msg(retired(be));
+        if (step == Step::Fused) {
+            auto r = fused(q, k, v, scale, act16, nullptr, st);
+            if (!is_ok(r)) return std::get<TensorError>(r);
+            auto& o = std::get<std::optional<Tensor>>(r);
+            if (o) return std::move(*o);
+        }
+        if (step == Step::Composed) composed_step = true;
     }
+    if (!composed_step) return msg("sdpa: every kernel of the route declined");
     // Step::Composed on the bf16-rounded operands under bf16 activations
     Tensor tq, tk, tv;
     const Tensor *pq = &q, *pk = &k, *pv = &v;
@@ -436,6 +455,44 @@ bool causal_flash_enabled() {
     return env;
 }
 
+Backend parse_backend(const std::string& v) {
+    if (v == "cublas") return Backend::Cublas;
+    if (v == "flash") return Backend::Flash;
+    if (v == "host") return Backend::Host;
+    if (v == "sparse") return Backend::Sparse;
+    return Backend::Dense;
+}
+Backend backend() {
+    if (g_backend_override) return *g_backend_override;
+    static const Backend env = [] {
+        const char* v = getenv("FASTVIDEO_SDPA");
+        std::string s = v ? v : "dense";
+        for (char& c : s) c = (char)tolower((unsigned char)c);
+        return parse_backend(s);
+    }();
+    return env;
+}
+void set_backend_override(std::optional<Backend> v) { g_backend_override = v; }
+
+Shape Shape::of(const std::vector<size_t>& q, const std::vector<size_t>& k, const std::vector<size_t>& v) {
+    Shape s;
+    s.sq = q.size() > 2 ? q[2] : 0;
+    s.sk = k.size() > 2 ? k[2] : 0;
+    if (q.size() == 4 && k.size() == 4 && k == std::vector<size_t>{q[0], q[1], k[2], q[3]} && v == k)
+        s.dims = Dims{q[0], q[1], q[2], k[2], q[3]};
+    return s;
+}
+
+std::vector<Step> dense_route(const Shape&, bool masked, Backend be) {
+    std::vector<Step> route;
+    if (!masked) {
+        if (be == Backend::Host || be == Backend::Sparse) return {Step::Retired};
+        if (be == Backend::Dense) route.push_back(Step::Fused);
+    }
+    route.push_back(Step::Composed);
+    return route;
+}
+
 Stats stats_snapshot() {
     Stats s;
     s.fused_launches = g_fused;
@@ -572,6 +629,26 @@ void fv_rt_set_bf16_activations(int v) {
     fv::rt::set_bf16_activations_override(v < 0 ? std::nullopt : std::optional<bool>(v != 0));
 }
 int fv_rt_bf16_activations(void) { return fv::rt::bf16_activations() ? 1 : 0; }
+
+int fv_rt_parse_backend(const char* v) { return (int)fv::rt::parse_backend(v ? v : ""); }
+int fv_rt_backend(void) { return (int)fv::rt::backend(); }
+void fv_rt_set_backend(int v) {
+    fv::rt::set_backend_override(v < 0 || v > 4 ? std::nullopt
+                                                : std::optional<fv::rt::Backend>((fv::rt::Backend)v));
+}
+int fv_rt_dense_route(const size_t* q_shape, const size_t* k_shape, const size_t* v_shape, int masked,
+                      int backend, int steps_out[4], size_t dims_out[5]) {
+    using namespace fv::rt;
+    if (!q_shape || !k_shape || !v_shape || !steps_out || backend < 0 || backend > 4) return -1;
+    const Shape s = Shape::of({q_shape, q_shape + 4}, {k_shape, k_shape + 4}, {v_shape, v_shape + 4});
+    if (dims_out) {
+        const Dims d = s.dims.value_or(Dims{0, 0, 0, 0, 0});
+        dims_out[0] = d.b, dims_out[1] = d.h, dims_out[2] = d.sq, dims_out[3] = d.sk, dims_out[4] = d.d;
+    }
+    const auto route = dense_route(s, masked != 0, (Backend)backend);
+    for (size_t i = 0; i < route.size() && i < 4; i++) steps_out[i] = (int)route[i];
+    return (int)route.size();
+}
 
 void fv_rt_stats(uint64_t out5[5]) {
     const auto s = fv::rt::stats_snapshot();

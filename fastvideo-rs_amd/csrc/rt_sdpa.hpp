@@ -103,6 +103,31 @@ void set_bf16_activations_override(std::optional<bool> v);
 // rt/sdpa_rule.rs `causal_flash_enabled`: FASTVIDEO_WAN_CAUSAL_FLASH, default on.
 bool causal_flash_enabled();
 
+// rt/sdpa_rule.rs:178-219 `Backend` / `parse_backend` / `backend`: FASTVIDEO_SDPA (lower-cased,
+// read once), overridable per thread. Anything but the four names below is the dense default.
+enum class Backend : int { Dense = 0, Cublas = 1, Flash = 2, Host = 3, Sparse = 4 };
+Backend parse_backend(const std::string& v);
+Backend backend();
+void set_backend_override(std::optional<Backend> v);
+
+// rt/sdpa_rule.rs:350-390 `Dims` / `Shape::of`: the lengths a dense call is chosen on, and the
+// five dims when k and v are both [b, h, sk, d] of q's [b, h, sq, d].
+struct Dims {
+    size_t b, h, sq, sk, d;
+};
+struct Shape {
+    size_t sq = 0, sk = 0;
+    std::optional<Dims> dims;
+    static Shape of(const std::vector<size_t>& q, const std::vector<size_t>& k, const std::vector<size_t>& v);
+};
+
+// rt/sdpa_rule.rs:392-437 `Step` / `dense_route`, with the NVIDIA alternates gone: an unmasked call
+// tries the fused gfx950 kernel and then the composed f32 kernel; FASTVIDEO_SDPA=cublas|flash (the
+// reference's f32-score kernels) go straight to the composed f32 kernel; host|sparse are retired and
+// refuse the call; a masked call is composed.
+enum class Step : int { Retired = 0, Fused = 1, Composed = 2 };
+std::vector<Step> dense_route(const Shape& shape, bool masked, Backend backend);
+
 // rt/sdpa.rs:141-164. Work is enqueued on `stream`; the result owns its buffer.
 Result<Tensor> sdpa(const Tensor& q, const Tensor& k, const Tensor& v, const Plan& plan,
                     hipStream_t stream);

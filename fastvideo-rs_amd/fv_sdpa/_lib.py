@@ -32,6 +32,10 @@ SIGNATURES = {
     "fv_rt_set_bf16_activations": (None, [C.c_int]),
     "fv_rt_bf16_activations": (C.c_int, []),
     "fv_rt_stats": (None, [_vp]),
+    "fv_rt_parse_backend": (C.c_int, [C.c_char_p]),
+    "fv_rt_backend": (C.c_int, []),
+    "fv_rt_set_backend": (None, [C.c_int]),
+    "fv_rt_dense_route": (C.c_int, [_vp, _vp, _vp, C.c_int, C.c_int, _vp, _vp]),
     "fv_vsa_topk_for": (_sz, [C.c_double, _sz]),
     "fv_vsa_tile_plan": (C.c_int, [_sz, _sz, _sz, _vp, _vp, _vp, _vp]),
     "fv_vsa_tile_mean": (C.c_int, [_vp, C.c_int, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_int, _vp]),

@@ -9,7 +9,8 @@ import torch
 
 from . import _lib
 
-__all__ = ["Plan", "BlockCausal", "VdnWindow", "sdpa", "with_bf16_act", "bf16_activations", "rt_stats", "TensorError"]
+__all__ = ["Plan", "BlockCausal", "VdnWindow", "sdpa", "with_bf16_act", "bf16_activations", "rt_stats", "TensorError",
+           "BACKENDS", "STEPS", "parse_backend", "backend", "with_backend", "shape_of", "dense_route"]
 
 
 class TensorError(RuntimeError):
@@ -208,3 +209,53 @@ def rt_stats():
     out = (C.c_uint64 * 5)()
     _lib.lib().fv_rt_stats(out)
     return dict(zip(("fused", "causal", "composed", "casts", "masks"), (int(x) for x in out)))
+
+
+# rt/sdpa_rule.rs:178-207 `Backend` and the collapsed `Step` (the NVIDIA alternates are gone)
+BACKENDS = ("dense", "cublas", "flash", "host", "sparse")
+STEPS = ("retired", "fused", "composed")
+
+
+def parse_backend(v):
+    """rt/sdpa_rule.rs:199-207: a FASTVIDEO_SDPA value -> backend name (unknown = "dense")."""
+    return BACKENDS[_lib.lib().fv_rt_parse_backend(str(v).encode())]
+
+
+def backend():
+    return BACKENDS[_lib.lib().fv_rt_backend()]
+
+
+@contextmanager
+def with_backend(name):
+    """Per-thread override of FASTVIDEO_SDPA for the calls inside the block."""
+    lib = _lib.lib()
+    lib.fv_rt_set_backend(BACKENDS.index(name))
+    try:
+        yield
+    finally:
+        lib.fv_rt_set_backend(-1)
+
+
+def _shape4(x):
+    x = tuple(int(i) for i in x)
+    if len(x) != 4:
+        raise TensorError("sdpa expects BHSD")
+    return (C.c_size_t * 4)(*x)
+
+
+def dense_route(q_shape, k_shape, v_shape, masked=False, backend_name="dense"):
+    """rt/sdpa_rule.rs:409-437: the kernels a dense call tries, in order."""
+    steps = (C.c_int * 4)()
+    n = _lib.lib().fv_rt_dense_route(_shape4(q_shape), _shape4(k_shape), _shape4(v_shape), int(bool(masked)),
+                                     BACKENDS.index(backend_name), steps, None)
+    if n < 0:
+        raise TensorError("dense_route: bad arguments")
+    return [STEPS[steps[i]] for i in range(n)]
+
+
+def shape_of(q_shape, k_shape, v_shape):
+    """rt/sdpa_rule.rs:373-390 `Shape::of`: (sq, sk, dims) with dims = (b, h, sq, sk, d) or None."""
+    steps, dims = (C.c_int * 4)(), (C.c_size_t * 5)()
+    _lib.lib().fv_rt_dense_route(_shape4(q_shape), _shape4(k_shape), _shape4(v_shape), 0, 0, steps, dims)
+    d = tuple(int(x) for x in dims)
+    return int(q_shape[2]), int(k_shape[2]), (d if any(d) else None)

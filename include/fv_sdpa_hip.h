@@ -119,6 +119,19 @@ int fv_rt_free(void* p, void* stream);
 /* rt/tensor.rs `with_bf16_act`: per-thread override of FASTVIDEO_BF16_ACT; v < 0 clears it. */
 void fv_rt_set_bf16_activations(int v);
 int fv_rt_bf16_activations(void);
+/* rt/sdpa_rule.rs:178-219 `Backend`, `parse_backend`, `backend`: FASTVIDEO_SDPA. 0 dense (the
+ * default and every unknown value), 1 cublas, 2 flash, 3 host, 4 sparse. fv_rt_set_backend is a
+ * per-thread override of the environment (v < 0 clears it). */
+int fv_rt_parse_backend(const char* v);
+int fv_rt_backend(void);
+void fv_rt_set_backend(int v);
+/* rt/sdpa_rule.rs:363-437 `Shape::of` + `dense_route` with the NVIDIA alternates removed. Shapes are
+ * rank 4. steps_out receives the route (0 retired: the call is refused; 1 the fused gfx950 kernel;
+ * 2 the composed f32 kernel), the return value is its length; dims_out (optional) = {b,h,sq,sk,d}
+ * when k and v are both [b,h,sk,d], else zeros. Route: unmasked dense -> {1, 2}; cublas / flash (the
+ * reference's f32-score kernels) -> {2}; host / sparse -> {0}; masked -> {2}. Host only. */
+int fv_rt_dense_route(const size_t* q_shape, const size_t* k_shape, const size_t* v_shape, int masked,
+                      int backend, int steps_out[4], size_t dims_out[5]);
 /* rt/stats.rs:27-72 analogue: {fused dense launches, block-causal launches, composed launches,
  * cast launches, dense masks materialised} since the library was loaded. */
 void fv_rt_stats(uint64_t out5[5]);

@@ -142,6 +142,31 @@ def test_dense_plan_reaches_the_fused_kernel(fv, oracle, act16, f32_in):
                   max_abs=2e-2 if act16 else 1e-2)
 
 
+def test_backend_setting_steers_the_dense_route(fv, oracle):
+    """FASTVIDEO_SDPA (rt/sdpa_rule.rs:199-219, 409-437; rt/sdpa.rs:225-246): cublas / flash take the
+    f32-score kernel instead of the fused one, host / sparse are retired and refuse the call."""
+    import torch
+
+    b, h, sq, sk, d = 1, 2, 130, 190, 128
+    announce("rt backend routes")
+    q, k, v = qkv(310, b * h, sq, sk, d)
+    tq, tk, tv = (dev(x.reshape(b, h, -1, d)).to(torch.bfloat16) for x in (q, k, v))
+    want = oracle.sdpa_composed(q, k, v)
+    for name in ("cublas", "flash"):
+        before = fv.rt_stats()
+        with fv.with_backend(name), fv.with_bf16_act(False):
+            got = fv.sdpa(tq, tk, tv, fv.Plan.dense(None))
+        after = fv.rt_stats()
+        assert after["fused"] == before["fused"] and after["composed"] == before["composed"] + 1
+        assert_parity(host(got).reshape(b * h, sq, d), want, f"rt_backend_{name}", max_abs=1e-5)
+    for name, needle in (("host", "retired"), ("sparse", "FASTVIDEO_VSA=1")):
+        with fv.with_backend(name), pytest.raises(fv.TensorError, match=needle):
+            fv.sdpa(tq, tk, tv, fv.Plan.dense(None))
+    before = fv.rt_stats()
+    fv.sdpa(tq, tk, tv, fv.Plan.dense(None))
+    assert fv.rt_stats()["fused"] == before["fused"] + 1
+
+
 def test_block_causal_and_kv_window_plans_at_d128(fv, oracle):
     import torch
 

@@ -77,3 +77,35 @@ def test_shard_ranges(oracle):
     assert fv_sdpa.shard_ranges(10, 2) == [(0, 5), (5, 5)]
     assert fv_sdpa.shard_ranges(11, 2) == [(0, 6), (6, 5)]
     assert fv_sdpa.shard_ranges(32760, 8) == oracle.shard_ranges(32760, 8)
+
+
+def test_backend_parses_like_the_reference():
+    # rt/sdpa_rule.rs:593-604
+    for v in ("dense", "cublas", "flash", "host", "sparse"):
+        assert fv_sdpa.parse_backend(v) == v
+    for v in ("", "fused", " cublas", "dense "):
+        assert fv_sdpa.parse_backend(v) == "dense", v
+    assert fv_sdpa.backend() == fv_sdpa.parse_backend(os.environ.get("FASTVIDEO_SDPA", "dense").lower())
+    with fv_sdpa.with_backend("cublas"):
+        assert fv_sdpa.backend() == "cublas"
+    assert fv_sdpa.backend() == fv_sdpa.parse_backend(os.environ.get("FASTVIDEO_SDPA", "dense").lower())
+
+
+def test_shapes_agree_only_when_k_and_v_match_q():
+    # rt/sdpa_rule.rs:624-651
+    assert fv_sdpa.shape_of((1, 2, 5, 64), (1, 2, 7, 64), (1, 2, 7, 64)) == (5, 7, (1, 2, 5, 7, 64))
+    assert fv_sdpa.shape_of((1, 2, 5, 64), (1, 2, 7, 64), (1, 2, 6, 64))[2] is None
+    assert fv_sdpa.shape_of((1, 2, 5, 64), (1, 3, 7, 64), (1, 3, 7, 64))[2] is None
+    assert fv_sdpa.shape_of((1, 2, 5, 64), (1, 2, 7, 32), (1, 2, 7, 32))[2] is None
+
+
+def test_dense_route_collapsed():
+    # rt/sdpa_rule.rs:409-437 without the cuDNN / cuBLAS / Sage / f32-flash steps
+    s = ((1, 12, 320, 128),) * 3
+    assert fv_sdpa.dense_route(*s) == ["fused", "composed"]
+    assert fv_sdpa.dense_route(*s, masked=True) == ["composed"]
+    for b in ("cublas", "flash"):
+        assert fv_sdpa.dense_route(*s, backend_name=b) == ["composed"]
+    for b in ("host", "sparse"):
+        assert fv_sdpa.dense_route(*s, backend_name=b) == ["retired"]
+        assert fv_sdpa.dense_route(*s, masked=True, backend_name=b) == ["composed"]   # masked calls never look
