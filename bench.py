@@ -100,6 +100,8 @@ def bench_vsa(args):
         "fine": timed(lambda: V.vsa_fine(qt, kt, vt, sel, ctx, scale), 10, 2)[2],
         "combine": timed(lambda: V.vsa_combine(sparse, coarse, gate, ctx, out=out), 10, 2)[2],
     }
+    # the whole op on operands a producer already wrote tile-ordered (no tile pass)
+    wall_t, avg_t, med_t = timed(lambda: V.vsa_attention_tiled(qt, kt, vt, gate, ctx, scale), args.steps, args.warmup)
     # the fine kernel alone on the selection the reference's own fine-kernel benchmark uses
     # (gpucheck kernels_attn.rs:199-208): tile (i + 7h + j) mod nb for j < topk, i.e. a band of
     # consecutive key tiles that neighbouring query tiles share almost entirely
@@ -118,6 +120,7 @@ def bench_vsa(args):
         "config": {"workload": desc, "H": h, "grid": list(grid), "tiles": nb, "topk": topk, "seq": seq, "d": d,
                    "inputs": "bf16 q/k/v/gate", "flops_per_call": flops},
         "whole_op_avg_ms": round(avg_ms, 4), "whole_op_median_ms": round(med_ms, 4),
+        "whole_op_tile_ordered_inputs_ms": {"avg": round(avg_t, 4), "median": round(med_t, 4), "wall": round(wall_t, 4)},
         "stages_median_ms": {k2: round(v2, 4) for k2, v2 in stages.items()},
         "roofline": {"bound": "mfma", "achieved": round(fine_tflops, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(fine_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::vsa_fine_kernel",
@@ -172,6 +175,14 @@ def bench_prep(args):
         "split_heads_bhsd (bf16)": (lambda: fv_sdpa.split_heads_bhsd(proj, 2 * width, heads, d), 2 * row),
         "merge_heads (bf16)": (lambda: fv_sdpa.merge_heads(o), 2 * row),
     }
+    # the same producers writing VSA's tile-slot order of the Wan 480p latent grid (21,30,52)
+    ctx = fv_sdpa.VsaCtx((21, 30, 52), 0.8, device=dev)
+    assert ctx.seq == seq
+    qt = torch.zeros((batch, heads, ctx.padded, d), device=dev, dtype=torch.bfloat16)
+    vt = torch.zeros_like(qt)
+    ops["qk_norm_rope_tiles (bf16, rope)"] = (
+        lambda: fv_sdpa.qk_norm_rope_tiles(proj, 0, heads, w, ctx, (cos, sin), out=qt), 2 * row + tables + width * 4)
+    ops["split_heads_tiles (bf16)"] = (lambda: fv_sdpa.split_heads_tiles(proj, 2 * width, heads, d, ctx, out=vt), 2 * row)
     res = {}
     for name, (fn, nbytes) in ops.items():
         wall, avg = timed(fn)

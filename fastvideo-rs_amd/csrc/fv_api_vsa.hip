@@ -153,7 +153,7 @@ void fv_sp_shard_ranges(size_t seq, size_t world, size_t* out) {
 int fv_vsa_tile_mean(const void* x, int x_is_bf16, const int32_t* slot_src, const int32_t* block_sizes,
                      float* out, size_t bh, size_t seq, size_t dim, size_t num_tiles, int round16,
                      void* stream) {
-    if (!x || !slot_src || !block_sizes || !out) return fv_invalid("vsa_tile_mean: null operand");
+    if (!x || !block_sizes || !out) return fv_invalid("vsa_tile_mean: null operand");
     if (bh == 0 || num_tiles == 0) return FV_OK;
     if (dim == 0 || dim % 4 != 0 || !fits_int(dim) || !fits_int(num_tiles) || bh > 65535)
         return fv_decline("vsa_tile_mean: needs dim % 4 == 0 and bh <= 65535");
@@ -257,18 +257,25 @@ size_t fv_vsa_workspace_bytes(size_t bh, size_t num_tiles, size_t topk, size_t d
     return vsa_layout(bh, num_tiles, topk, dim).total;
 }
 
-int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf16, const void* gate,
-                     int gate_is_bf16, const int32_t* slot_src, const int32_t* block_sizes, float* out,
-                     void* workspace, size_t workspace_bytes, uint32_t* selected_out, size_t bh,
-                     size_t seq, size_t num_tiles, size_t topk, size_t dim, float scale, void* stream) {
+// The whole op. tiled != 0: q/k/v are bf16 [bh, num_tiles*64, 128] already in tile-slot order (zero
+// padding slots), so the tile means read them in place and the tile pass is skipped.
+static int vsa_attention_common(const void* q, const void* k, const void* v, int qkv_is_bf16, int tiled,
+                                const void* gate, int gate_is_bf16, const int32_t* slot_src,
+                                const int32_t* block_sizes, float* out, void* workspace,
+                                size_t workspace_bytes, uint32_t* selected_out, size_t bh, size_t seq,
+                                size_t num_tiles, size_t topk, size_t dim, float scale, void* stream) {
     if (!q || !k || !v || !slot_src || !block_sizes || !out || !workspace)
         return fv_invalid("vsa_attention: null operand");
     if (topk < 1) topk = 1;                 // rt/vsa.rs:373 `topk.clamp(1, nb)`
     if (topk > num_tiles) topk = num_tiles;
     if (dim != 128 || num_tiles == 0 || num_tiles > kTopkMaxN || bh == 0 || bh > 65535)
         return fv_decline("vsa_attention: needs dim == 128, 1 <= num_tiles <= 4096, 1 <= bh <= 65535");
+    const size_t padded = num_tiles * kTile;
+    if (!(scale > 0.0f) || !(scale < 3.0e38f) || !fits_int(padded) || bh * num_tiles > (size_t)INT_MAX / 2)
+        return fv_decline("vsa_attention: needs a finite scale > 0 and a tile count that fits one launch");
     const VsaWorkspace w = vsa_layout(bh, num_tiles, topk, dim);
-    if (workspace_bytes < w.total) return fv_invalid("vsa_attention: workspace too small (fv_vsa_workspace_bytes)");
+    const size_t need = tiled ? w.qt : w.total;   // the tile-ordered copies are the tail of the layout
+    if (workspace_bytes < need) return fv_invalid("vsa_attention: workspace too small (fv_vsa_workspace_bytes)");
     if (((uintptr_t)workspace & 255) != 0) return fv_invalid("vsa_attention: workspace must be 256-byte aligned");
     char* ws = (char*)workspace;
     float* qc = (float*)(ws + w.qc);
@@ -277,27 +284,38 @@ int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf1
     float* scores = (float*)(ws + w.scores);
     float* coarse = (float*)(ws + w.coarse);
     uint32_t* sel = selected_out ? selected_out : (uint32_t*)(ws + w.selected);
-    uint16_t* qt = (uint16_t*)(ws + w.qt);
-    uint16_t* kt = (uint16_t*)(ws + w.kt);
-    uint16_t* vt = (uint16_t*)(ws + w.vt);
-    const size_t padded = num_tiles * kTile;
+    const uint16_t *qt = (const uint16_t*)q, *kt = (const uint16_t*)k, *vt = (const uint16_t*)v;
+    // tile-ordered input: identity slot map (null), rows per bh = padded
+    const int32_t* mean_map = tiled ? nullptr : slot_src;
+    const size_t mean_rows = tiled ? padded : seq;
+    const int in16 = tiled ? 1 : qkv_is_bf16;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e;
     int rc;
     // 1. tile means (rt/vsa.rs:378-384)
-    if ((rc = fv_vsa_tile_mean(q, qkv_is_bf16, slot_src, block_sizes, qc, bh, seq, dim, num_tiles, 0, stream))) return rc;
-    if ((rc = fv_vsa_tile_mean(k, qkv_is_bf16, slot_src, block_sizes, kc, bh, seq, dim, num_tiles, 0, stream))) return rc;
-    if ((rc = fv_vsa_tile_mean(v, qkv_is_bf16, slot_src, block_sizes, vc, bh, seq, dim, num_tiles, 0, stream))) return rc;
+    for (int i = 0; i < 3; i++) {
+        const void* x = i == 0 ? q : (i == 1 ? k : v);
+        float* m = i == 0 ? qc : (i == 1 ? kc : vc);
+        e = fv_internal_launch_tile_mean(x, in16, mean_map, block_sizes, m, bh, mean_rows, (int)dim, (int)num_tiles,
+                                         0, st);
+        if (e != hipSuccess) return fv_fail_hip(e, "vsa_tile_mean");
+    }
     // 2. coarse attention over tiles; raw scores kept for the selection (rt/vsa.rs:385-394)
     if ((rc = fv_vsa_coarse(qc, kc, vc, scores, coarse, bh, num_tiles, dim, scale, stream))) return rc;
     // 3. top-k tiles per query tile (rt/vsa.rs:398-400)
     if ((rc = fv_vsa_topk(scores, sel, bh * num_tiles, num_tiles, topk, stream))) return rc;
     // 4. fine stage on tile-ordered bf16 copies (rt/vsa.rs:406-414)
-    if ((rc = fv_vsa_tile_qkv(q, qkv_is_bf16, slot_src, qt, bh, seq, padded, dim, stream))) return rc;
-    if ((rc = fv_vsa_tile_qkv(k, qkv_is_bf16, slot_src, kt, bh, seq, padded, dim, stream))) return rc;
-    if ((rc = fv_vsa_tile_qkv(v, qkv_is_bf16, slot_src, vt, bh, seq, padded, dim, stream))) return rc;
+    if (!tiled) {
+        uint16_t* tq = (uint16_t*)(ws + w.qt);
+        uint16_t* tk = (uint16_t*)(ws + w.kt);
+        uint16_t* tv = (uint16_t*)(ws + w.vt);
+        if ((rc = fv_vsa_tile_qkv(q, qkv_is_bf16, slot_src, tq, bh, seq, padded, dim, stream))) return rc;
+        if ((rc = fv_vsa_tile_qkv(k, qkv_is_bf16, slot_src, tk, bh, seq, padded, dim, stream))) return rc;
+        if ((rc = fv_vsa_tile_qkv(v, qkv_is_bf16, slot_src, tv, bh, seq, padded, dim, stream))) return rc;
+        qt = tq, kt = tk, vt = tv;
+    }
     // 5. out = coarse * gate + sparse, back in token order: fused into the fine kernel's epilogue
     //    (no f32 sparse buffer: 2 x 200 MB of traffic and 200 MB of workspace less at Wan 480p)
-    if (!(scale > 0.0f) || !(scale < 3.0e38f) || !fits_int(padded) || bh * num_tiles > (size_t)INT_MAX / 2)
-        return fv_decline("vsa_attention: needs a finite scale > 0 and a tile count that fits one launch");
     fv::VsaFineParams p;
     p.qt = qt;
     p.kt = kt;
@@ -318,8 +336,24 @@ int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf1
     p.gate_is_bf16 = gate_is_bf16;
     p.slot_src = slot_src;
     p.seq = (long)seq;
-    hipError_t e = fv_internal_launch_fine(&p, (hipStream_t)stream);
+    e = fv_internal_launch_fine(&p, st);
     return e == hipSuccess ? FV_OK : fv_fail_hip(e, "vsa_fine (fused combine)");
+}
+
+int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf16, const void* gate,
+                     int gate_is_bf16, const int32_t* slot_src, const int32_t* block_sizes, float* out,
+                     void* workspace, size_t workspace_bytes, uint32_t* selected_out, size_t bh,
+                     size_t seq, size_t num_tiles, size_t topk, size_t dim, float scale, void* stream) {
+    return vsa_attention_common(q, k, v, qkv_is_bf16, 0, gate, gate_is_bf16, slot_src, block_sizes, out, workspace,
+                                workspace_bytes, selected_out, bh, seq, num_tiles, topk, dim, scale, stream);
+}
+
+int fv_vsa_attention_tiled(const uint16_t* qt, const uint16_t* kt, const uint16_t* vt, const void* gate,
+                           int gate_is_bf16, const int32_t* slot_src, const int32_t* block_sizes, float* out,
+                           void* workspace, size_t workspace_bytes, uint32_t* selected_out, size_t bh,
+                           size_t seq, size_t num_tiles, size_t topk, size_t dim, float scale, void* stream) {
+    return vsa_attention_common(qt, kt, vt, 1, 1, gate, gate_is_bf16, slot_src, block_sizes, out, workspace,
+                                workspace_bytes, selected_out, bh, seq, num_tiles, topk, dim, scale, stream);
 }
 
 }  // extern "C"

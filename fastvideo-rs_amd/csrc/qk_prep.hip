@@ -77,7 +77,7 @@ template <bool X16, bool W16, bool ROUND16, int NC>
 __global__ __launch_bounds__(256) void qk_norm_rope_bhsd_kernel(
     const void* __restrict__ src, const void* __restrict__ w, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, void* __restrict__ out, long rows, int seq, int heads, int d,
-    long src_width, long col_off, float eps) {
+    long src_width, long col_off, float eps, const unsigned* __restrict__ row_map, long out_rows) {
 #pragma clang fp contract(off)
     const int lane = threadIdx.x & 63;
     const long row = (long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
@@ -114,6 +114,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_bhsd_kernel(
     ss = wave_sum(ss);
     const float inv = 1.0f / __builtin_sqrtf(ss / (float)width + eps);
 
+    // row_map: the head planes are [out_rows, d] and token s lands in row row_map[s] (the VSA
+    // tile-slot order); without it the planes are [seq, d] in token order.
+    const size_t orow = row_map ? row_map[s] : (unsigned)s;
+    if (orow >= (size_t)out_rows) return;   // a slot outside the plane: nothing is written
     const bool rope = cos_t != nullptr;
     // With d/8 dividing 64 every chunk of a lane sits at the same offset p inside its head,
     // so the lane's 8 cos / 8 sin values are loaded once per row instead of once per head.
@@ -156,7 +160,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_bhsd_kernel(
                 r[i + 1] = ROUND16 ? (x2 * cv + x1 * sv) : (x1 * sv + x2 * cv);
             }
         }
-        const size_t o = (((size_t)b * heads + h) * seq + s) * d + p;
+        const size_t o = (((size_t)b * heads + h) * out_rows + orow) * d + p;
         if constexpr (ROUND16) {
             *reinterpret_cast<u32x4*>((unsigned short*)out + o) = pack_bf16x8(r);
         } else {
@@ -178,10 +182,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_bhsd_kernel(
 }
 
 // Both permutes move 16-byte units; `du` = units per head row (d * elem / 16).
-// split: out[((b*heads + h)*seq + s)*du + u] = src[(b*seq + s)*wu + cu + h*du + u]
+// split: out[((b*heads + h)*seq + s)*du + u] = src[(b*seq + s)*wu + cu + h*du + u]; with a row map
+// the planes are [out_rows, du] and token s lands in row row_map[s].
 __global__ __launch_bounds__(256) void split_heads_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ out,
                                                           size_t n, size_t seq, size_t heads, size_t du,
-                                                          size_t wu, size_t cu) {
+                                                          size_t wu, size_t cu,
+                                                          const unsigned* __restrict__ row_map, size_t out_rows) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     const size_t u = i % du;
@@ -189,7 +195,13 @@ __global__ __launch_bounds__(256) void split_heads_kernel(const u32x4* __restric
     const size_t s = t % seq;
     t /= seq;
     const size_t h = t % heads, b = t / heads;
-    out[i] = src[(b * seq + s) * wu + cu + h * du + u];
+    size_t o = i;
+    if (row_map) {
+        const size_t r = row_map[s];
+        if (r >= out_rows) return;   // a slot outside the plane: nothing is written
+        o = ((b * heads + h) * out_rows + r) * du + u;
+    }
+    out[o] = src[(b * seq + s) * wu + cu + h * du + u];
 }
 
 // merge: out[(b*seq + s)*heads*du + h*du + u] = src[((b*heads + h)*seq + s)*du + u]
@@ -207,17 +219,18 @@ __global__ __launch_bounds__(256) void merge_heads_kernel(const u32x4* __restric
 template <bool X16, bool W16, bool R16, int NC>
 void launch_qk_nc(dim3 grid, hipStream_t st, const void* src, const void* w, const float* cos_t,
                   const float* sin_t, void* out, long rows, int seq, int heads, int d, long src_width,
-                  long col_off, float eps) {
+                  long col_off, float eps, const unsigned* row_map, long out_rows) {
     hipLaunchKernelGGL((qk_norm_rope_bhsd_kernel<X16, W16, R16, NC>), grid, dim3(256), 0, st, src, w, cos_t, sin_t,
-                       out, rows, seq, heads, d, src_width, col_off, eps);
+                       out, rows, seq, heads, d, src_width, col_off, eps, row_map, out_rows);
 }
 
 template <bool X16, bool W16, bool R16>
 void launch_qk_r(const void* src, const void* w, const float* cos_t, const float* sin_t, void* out, long rows,
-                 int seq, int heads, int d, long src_width, long col_off, float eps, hipStream_t st) {
+                 int seq, int heads, int d, long src_width, long col_off, float eps, const unsigned* row_map,
+                 long out_rows, hipStream_t st) {
     const dim3 grid((unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock));
     const int per_lane = (heads * d / 8 + 63) / 64;   // 16-byte chunks per lane
-#define FV_QK_ARGS grid, st, src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps
+#define FV_QK_ARGS grid, st, src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, row_map, out_rows
     if (per_lane <= 2) launch_qk_nc<X16, W16, R16, 2>(FV_QK_ARGS);
     else if (per_lane <= 3) launch_qk_nc<X16, W16, R16, 3>(FV_QK_ARGS);        // 12 heads x 128
     else if (per_lane <= 6) launch_qk_nc<X16, W16, R16, 6>(FV_QK_ARGS);
@@ -229,9 +242,13 @@ void launch_qk_r(const void* src, const void* w, const float* cos_t, const float
 template <bool X16, bool W16>
 hipError_t launch_qk(int round16, const void* src, const void* w, const float* cos_t, const float* sin_t,
                      void* out, long rows, int seq, int heads, int d, long src_width, long col_off,
-                     float eps, hipStream_t st) {
-    if (round16) launch_qk_r<X16, W16, true>(src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, st);
-    else launch_qk_r<X16, W16, false>(src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, st);
+                     float eps, const unsigned* row_map, long out_rows, hipStream_t st) {
+    if (round16)
+        launch_qk_r<X16, W16, true>(src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, row_map,
+                                    out_rows, st);
+    else
+        launch_qk_r<X16, W16, false>(src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps,
+                                     row_map, out_rows, st);
     return hipGetLastError();
 }
 
@@ -240,10 +257,11 @@ hipError_t launch_qk(int round16, const void* src, const void* w, const float* c
 
 extern "C" {
 
-int fv_qk_norm_rope_bhsd(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
-                         const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
-                         size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
-                         size_t col_off, float eps, void* stream) {
+static int qk_norm_rope_common(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
+                               const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
+                               size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
+                               size_t col_off, float eps, const uint32_t* row_map, size_t out_rows,
+                               void* stream) {
     if (!src || !w || !out) return fv_invalid("qk_norm_rope: null operand");
     if ((cos_t == nullptr) != (sin_t == nullptr)) return fv_invalid("qk_norm_rope: one rope table without the other");
     if (batch == 0 || seq == 0) return FV_OK;
@@ -252,28 +270,45 @@ int fv_qk_norm_rope_bhsd(const void* src, int src_is_bf16, const void* w, int w_
     // 16-byte lane chunks: 8 elements, never straddling a head, aligned in the source row
     if (d % 8 != 0 || col_off % 8 != 0 || src_width % 8 != 0)
         return fv_decline("qk_norm_rope: d, col_off and src_width must be multiples of 8");
-    if (batch * seq > (size_t)INT_MAX || seq > (size_t)INT_MAX || heads * d > (size_t)INT_MAX / 2)
+    if (batch * seq > (size_t)INT_MAX || seq > (size_t)INT_MAX || heads * d > (size_t)INT_MAX / 2 ||
+        out_rows > (size_t)INT_MAX)
         return fv_decline("qk_norm_rope: too large for one launch");
     const long rows = (long)(batch * seq);
     hipStream_t st = (hipStream_t)stream;
     hipError_t e;
-    if (src_is_bf16 && w_is_bf16)
-        e = fv::launch_qk<true, true>(out_is_bf16, src, w, cos_t, sin_t, out, rows, (int)seq, (int)heads, (int)d,
-                                      (long)src_width, (long)col_off, eps, st);
-    else if (src_is_bf16)
-        e = fv::launch_qk<true, false>(out_is_bf16, src, w, cos_t, sin_t, out, rows, (int)seq, (int)heads, (int)d,
-                                       (long)src_width, (long)col_off, eps, st);
-    else if (w_is_bf16)
-        e = fv::launch_qk<false, true>(out_is_bf16, src, w, cos_t, sin_t, out, rows, (int)seq, (int)heads, (int)d,
-                                       (long)src_width, (long)col_off, eps, st);
-    else
-        e = fv::launch_qk<false, false>(out_is_bf16, src, w, cos_t, sin_t, out, rows, (int)seq, (int)heads, (int)d,
-                                        (long)src_width, (long)col_off, eps, st);
+#define FV_QK_CALL(X16, W16)                                                                                  \
+    fv::launch_qk<X16, W16>(out_is_bf16, src, w, cos_t, sin_t, out, rows, (int)seq, (int)heads, (int)d,        \
+                            (long)src_width, (long)col_off, eps, row_map, (long)out_rows, st)
+    if (src_is_bf16 && w_is_bf16) e = FV_QK_CALL(true, true);
+    else if (src_is_bf16) e = FV_QK_CALL(true, false);
+    else if (w_is_bf16) e = FV_QK_CALL(false, true);
+    else e = FV_QK_CALL(false, false);
+#undef FV_QK_CALL
     return e == hipSuccess ? FV_OK : fv_fail_hip(e, "qk_norm_rope_bhsd");
 }
 
-int fv_split_heads_bhsd(const void* src, void* out, int is_bf16, size_t batch, size_t seq, size_t heads,
-                        size_t d, size_t src_width, size_t col_off, void* stream) {
+int fv_qk_norm_rope_bhsd(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
+                         const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
+                         size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
+                         size_t col_off, float eps, void* stream) {
+    return qk_norm_rope_common(src, src_is_bf16, w, w_is_bf16, cos_t, sin_t, out, out_is_bf16, batch, seq, heads, d,
+                               src_width, col_off, eps, nullptr, seq, stream);
+}
+
+int fv_qk_norm_rope_tiles(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
+                          const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
+                          size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
+                          size_t col_off, float eps, const uint32_t* token_slot, size_t padded,
+                          void* stream) {
+    if (!token_slot) return fv_invalid("qk_norm_rope_tiles: null token_slot");
+    if (padded < seq) return fv_invalid("qk_norm_rope_tiles: padded < seq");
+    return qk_norm_rope_common(src, src_is_bf16, w, w_is_bf16, cos_t, sin_t, out, out_is_bf16, batch, seq, heads, d,
+                               src_width, col_off, eps, token_slot, padded, stream);
+}
+
+static int split_heads_common(const void* src, void* out, int is_bf16, size_t batch, size_t seq, size_t heads,
+                              size_t d, size_t src_width, size_t col_off, const uint32_t* row_map,
+                              size_t out_rows, void* stream) {
     if (!src || !out) return fv_invalid("split_heads: null operand");
     if (col_off + heads * d > src_width) return fv_invalid("split_heads: columns outside the projection");
     const size_t per16 = is_bf16 ? 8 : 4;
@@ -285,9 +320,23 @@ int fv_split_heads_bhsd(const void* src, void* out, int is_bf16, size_t batch, s
     if (blocks > (size_t)INT_MAX) return fv_decline("split_heads: too large for one launch");
     hipLaunchKernelGGL(fv::split_heads_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        (const fv::u32x4*)src, (fv::u32x4*)out, n, seq, heads, du, src_width / per16,
-                       col_off / per16);
+                       col_off / per16, row_map, out_rows);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FV_OK : fv_fail_hip(e, "split_heads_bhsd");
+}
+
+int fv_split_heads_bhsd(const void* src, void* out, int is_bf16, size_t batch, size_t seq, size_t heads,
+                        size_t d, size_t src_width, size_t col_off, void* stream) {
+    return split_heads_common(src, out, is_bf16, batch, seq, heads, d, src_width, col_off, nullptr, seq, stream);
+}
+
+int fv_split_heads_tiles(const void* src, void* out, int is_bf16, size_t batch, size_t seq, size_t heads,
+                         size_t d, size_t src_width, size_t col_off, const uint32_t* token_slot, size_t padded,
+                         void* stream) {
+    if (!token_slot) return fv_invalid("split_heads_tiles: null token_slot");
+    if (padded < seq) return fv_invalid("split_heads_tiles: padded < seq");
+    return split_heads_common(src, out, is_bf16, batch, seq, heads, d, src_width, col_off, token_slot, padded,
+                              stream);
 }
 
 int fv_merge_heads(const void* src, void* out, int is_bf16, size_t batch, size_t heads, size_t seq, size_t d,

@@ -24,7 +24,9 @@ __global__ __launch_bounds__(256) void vsa_tile_mean_kernel(
     const long bh = blockIdx.y;
     if (tile >= num_tiles) return;
     const int n = block_sizes[tile];
-    const int* src = slot_src + (long)tile * kTileElems;
+    // slot_src == null: x is already tile-ordered, slot j of the tile is row tile*64 + j
+    const int* src = slot_src ? slot_src + (long)tile * kTileElems : nullptr;
+    const long row0 = (long)tile * kTileElems;
     float* ob = out + (bh * num_tiles + tile) * (long)dim;
     auto load_tok = [&](long tok, int d0) -> f32x4 {
         f32x4 v;
@@ -51,14 +53,14 @@ __global__ __launch_bounds__(256) void vsa_tile_mean_kernel(
         for (; j + 8 <= n; j += 8) {
             f32x4 v[8];
 #pragma unroll
-            for (int u = 0; u < 8; u++) v[u] = load_tok(src[j + u], d0);
+            for (int u = 0; u < 8; u++) v[u] = load_tok(src ? src[j + u] : row0 + j + u, d0);
 #pragma unroll
             for (int u = 0; u < 8; u++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) acc[e] = __fadd_rn(acc[e], v[u][e]);
         }
         for (; j < n; j++) {
-            const f32x4 v = load_tok(src[j], d0);
+            const f32x4 v = load_tok(src ? src[j] : row0 + j, d0);
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[e] = __fadd_rn(acc[e], v[e]);
         }

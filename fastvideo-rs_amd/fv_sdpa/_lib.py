@@ -48,6 +48,8 @@ SIGNATURES = {
     "fv_vsa_workspace_bytes": (_sz, [_sz, _sz, _sz, _sz]),
     "fv_vsa_attention": (C.c_int, [_vp, _vp, _vp, C.c_int, _vp, C.c_int, _vp, _vp, _vp, _vp, _sz, _vp,
                                    _sz, _sz, _sz, _sz, _sz, C.c_float, _vp]),
+    "fv_vsa_attention_tiled": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _vp, _vp, _vp, _vp, _sz, _vp,
+                                         _sz, _sz, _sz, _sz, _sz, C.c_float, _vp]),
     "fv_block_causal_allows": (C.c_int, [_sz, _sz, _sz, _sz, _sz]),
     "fv_block_causal_dense_mask": (None, [_sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_block_causal_for": (C.c_int, [_sz, C.c_longlong, _sz, _vp]),
@@ -60,6 +62,9 @@ SIGNATURES = {
                                        _sz, C.c_float, _vp]),
     "fv_split_heads_bhsd": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_merge_heads": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _vp]),
+    "fv_qk_norm_rope_tiles": (C.c_int, [_vp, C.c_int, _vp, C.c_int, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz,
+                                        _sz, C.c_float, _vp, _sz, _vp]),
+    "fv_split_heads_tiles": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz, _sz, _vp, _sz, _vp]),
 }
 
 _lib = None

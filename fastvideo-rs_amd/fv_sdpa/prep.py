@@ -6,7 +6,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["qk_norm_rope_bhsd", "split_heads_bhsd", "merge_heads"]
+__all__ = ["qk_norm_rope_bhsd", "split_heads_bhsd", "merge_heads", "qk_norm_rope_tiles", "split_heads_tiles"]
 
 
 def _stream():
@@ -23,10 +23,14 @@ def _is16(t, name):
     raise ValueError(f"{name}: want f32 or bf16")
 
 
-def qk_norm_rope_bhsd(proj, col_off, heads, weight, rope=None, eps=1e-6, out_bf16=None):
+def qk_norm_rope_bhsd(proj, col_off, heads, weight, rope=None, eps=1e-6, out_bf16=None, tiles=None, out=None):
     """proj [batch, seq, width] -> [batch, heads, seq, d]. out_bf16 (default: proj is bf16)
-    selects the bf16 kernel with its rounding points; otherwise the f32 op."""
+    selects the bf16 kernel with its rounding points; otherwise the f32 op. `tiles` (a VsaCtx): the
+    head planes are written in the plan's tile-slot order, [batch, heads, padded, d], padding zero
+    (`out`: a buffer from an earlier call, whose padding rows are zero already)."""
     batch, seq, width = proj.shape
+    if tiles is not None and seq != tiles.seq:
+        raise ValueError(f"qk norm: proj has {seq} tokens, the tile plan {tiles.seq}")
     if heads == 0 or weight.numel() % heads or col_off + weight.numel() > width:
         raise ValueError("qk norm: weight / columns")
     d = weight.numel() // heads
@@ -40,11 +44,43 @@ def qk_norm_rope_bhsd(proj, col_off, heads, weight, rope=None, eps=1e-6, out_bf1
             raise ValueError("qk norm: rope needs an even head dim")
     x16, w16 = _is16(proj, "proj"), _is16(weight, "weight")
     out_bf16 = bool(x16) if out_bf16 is None else bool(out_bf16)
-    out = torch.empty((batch, heads, seq, d), device=proj.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    odt = torch.bfloat16 if out_bf16 else torch.float32
+    if tiles is not None:
+        if out is None:
+            out = torch.zeros((batch, heads, tiles.padded, d), device=proj.device, dtype=odt)
+        elif tuple(out.shape) != (batch, heads, tiles.padded, d) or out.dtype != odt or not out.is_contiguous():
+            raise ValueError("qk norm: out must be a contiguous [batch, heads, padded, d] tensor of the output type")
+        _lib.check(_lib.lib().fv_qk_norm_rope_tiles(proj.data_ptr(), x16, weight.data_ptr(), w16,
+                                                    cos.data_ptr() if cos is not None else None,
+                                                    sin.data_ptr() if sin is not None else None, out.data_ptr(),
+                                                    int(out_bf16), batch, seq, heads, d, width, col_off, eps,
+                                                    tiles.token_slot.data_ptr(), tiles.padded, _stream()))
+        return out
+    out = torch.empty((batch, heads, seq, d), device=proj.device, dtype=odt)
     _lib.check(_lib.lib().fv_qk_norm_rope_bhsd(proj.data_ptr(), x16, weight.data_ptr(), w16,
                                                cos.data_ptr() if cos is not None else None,
                                                sin.data_ptr() if sin is not None else None, out.data_ptr(),
                                                int(out_bf16), batch, seq, heads, d, width, col_off, eps, _stream()))
+    return out
+
+
+def qk_norm_rope_tiles(proj, col_off, heads, weight, ctx, rope=None, eps=1e-6, out_bf16=None, out=None):
+    """`qk_norm_rope_bhsd` writing VSA's tile-slot order directly (ctx: a VsaCtx)."""
+    return qk_norm_rope_bhsd(proj, col_off, heads, weight, rope, eps, out_bf16, tiles=ctx, out=out)
+
+
+def split_heads_tiles(proj, col_off, heads, d, ctx, out=None):
+    """`split_heads_bhsd` writing VSA's tile-slot order: [batch, heads, padded, d], padding zero."""
+    batch, seq, width = proj.shape
+    if seq != ctx.seq:
+        raise ValueError(f"split heads: proj has {seq} tokens, the tile plan {ctx.seq}")
+    is16 = _is16(proj, "proj")
+    if out is None:
+        out = torch.zeros((batch, heads, ctx.padded, d), device=proj.device, dtype=proj.dtype)
+    elif tuple(out.shape) != (batch, heads, ctx.padded, d) or out.dtype != proj.dtype or not out.is_contiguous():
+        raise ValueError("split heads: out must be a contiguous [batch, heads, padded, d] tensor of proj's type")
+    _lib.check(_lib.lib().fv_split_heads_tiles(proj.data_ptr(), out.data_ptr(), is16, batch, seq, heads, d, width,
+                                               col_off, ctx.token_slot.data_ptr(), ctx.padded, _stream()))
     return out
 
 

@@ -13,7 +13,7 @@ TILE = (4, 4, 4)
 TILE_ELEMS = 64
 
 __all__ = ["TILE", "TILE_ELEMS", "topk_for", "TilePlan", "VsaCtx", "vsa_tile_mean", "vsa_coarse", "vsa_topk",
-           "vsa_tile_qkv", "vsa_fine", "vsa_combine", "vsa_attention_device", "block_causal_allows",
+           "vsa_tile_qkv", "vsa_fine", "vsa_combine", "vsa_attention_device", "vsa_attention_tiled", "block_causal_allows",
            "block_causal_dense_mask", "block_causal_for", "shard_ranges"]
 
 
@@ -57,6 +57,8 @@ class VsaCtx:
         self.topk = topk_for(sparsity, self.plan.num_tiles)
         self.seq = self.plan.seq
         self.slot_src = torch.from_numpy(self.plan.slot_src).to(device)
+        self.token_slot = torch.from_numpy(self.plan.token_slot.astype(np.int32)).to(device)   # u32 bits
+        self.padded = self.plan.padded
         self.block_sizes = torch.from_numpy(self.plan.block_sizes).to(device)
 
     @property
@@ -77,12 +79,14 @@ def _chk(t, name, dtypes=(torch.float32, torch.bfloat16)):
         raise ValueError(f"{name}: want a contiguous CUDA tensor of {dtypes}")
 
 
-def vsa_tile_mean(x, ctx, round16=False):
+def vsa_tile_mean(x, ctx, round16=False, tiled=False):
+    """`tiled`: x is already in tile-slot order, [bh, padded, dim]."""
     _chk(x, "x")
     bh, seq, dim = x.shape
-    assert seq == ctx.seq
+    assert seq == (ctx.padded if tiled else ctx.seq)
     out = torch.empty((bh, ctx.num_tiles, dim), device=x.device, dtype=torch.float32)
-    _lib.check(_lib.lib().fv_vsa_tile_mean(x.data_ptr(), _is16(x), ctx.slot_src.data_ptr(), ctx.block_sizes.data_ptr(),
+    _lib.check(_lib.lib().fv_vsa_tile_mean(x.data_ptr(), _is16(x), None if tiled else ctx.slot_src.data_ptr(),
+                                           ctx.block_sizes.data_ptr(),
                                            out.data_ptr(), bh, seq, dim, ctx.num_tiles, int(round16), _stream()))
     return out
 
@@ -180,6 +184,35 @@ def vsa_attention_device(q, k, v, gate, ctx, scale, topk=None, return_selected=F
                                            ctx.block_sizes.data_ptr(), out.data_ptr(), ws.data_ptr(), nbytes,
                                            sel.data_ptr() if sel is not None else None, bh, seq, nb, topk, dim, scale,
                                            _stream()))
+    return (out, sel) if return_selected else out
+
+
+def vsa_attention_tiled(qt, kt, vt, gate, ctx, scale, topk=None, return_selected=False):
+    """`vsa_attention_device` on q/k/v that a producer already wrote tile-ordered:
+    qt/kt/vt bf16 [bh, padded, 128] with zero padding slots (`qk_norm_rope_tiles`, `split_heads_tiles`);
+    gate and out stay in token order. Same result, bit for bit, as `vsa_attention_device` on the
+    token-ordered bf16 tensors; the tile pass and its three buffers are not needed."""
+    for n, t in (("qt", qt), ("kt", kt), ("vt", vt)):
+        _chk(t, n, (torch.bfloat16,))
+    bh, padded, dim = qt.shape
+    if not (qt.shape == kt.shape == vt.shape) or padded != ctx.padded:
+        raise ValueError(f"vsa: tile-ordered q, k, v must be [bh, {ctx.padded}, dim]")
+    if gate is not None:
+        _chk(gate, "gate")
+        if tuple(gate.shape) != (bh, ctx.seq, dim):
+            raise ValueError("vsa: gate must be [bh, seq, dim] in token order")
+    nb = ctx.num_tiles
+    topk = min(max(int(ctx.topk if topk is None else topk), 1), nb)
+    out = torch.empty((bh, ctx.seq, dim), device=qt.device, dtype=torch.float32)
+    nbytes = int(_lib.lib().fv_vsa_workspace_bytes(bh, nb, topk, dim))
+    ws = torch.empty(nbytes, device=qt.device, dtype=torch.uint8)
+    sel = torch.empty((bh, nb, topk), device=qt.device, dtype=torch.int32) if return_selected else None
+    _lib.check(_lib.lib().fv_vsa_attention_tiled(qt.data_ptr(), kt.data_ptr(), vt.data_ptr(),
+                                                 gate.data_ptr() if gate is not None else None,
+                                                 _is16(gate) if gate is not None else 0, ctx.slot_src.data_ptr(),
+                                                 ctx.block_sizes.data_ptr(), out.data_ptr(), ws.data_ptr(), nbytes,
+                                                 sel.data_ptr() if sel is not None else None, bh, ctx.seq, nb, topk,
+                                                 dim, scale, _stream()))
     return (out, sel) if return_selected else out
 
 

@@ -152,7 +152,8 @@ int fv_vsa_tile_plan(size_t t, size_t h, size_t w, size_t dims_out[5], int32_t* 
 /* kernels/core.cu:550-570 `vsa_tile_mean`, kernels/attn3.cu:208-226 `vsa_tile_mean_b16`
  * (rt/ops.rs:868-872): out[bh, tile, :] = mean of the tile's real tokens, f32 sum in slot
  * order then / n. x is f32 or bf16 bits [bh, seq, dim]; round16 pools bf16-rounded values
- * of an f32 x. dim % 4 == 0. */
+ * of an f32 x. dim % 4 == 0. slot_src NULL: x is already tile-ordered, [bh, num_tiles*64, dim]
+ * with seq = num_tiles*64 (slot j of a tile is its row j). */
 int fv_vsa_tile_mean(const void* x, int x_is_bf16, const int32_t* slot_src, const int32_t* block_sizes,
                      float* out, size_t bh, size_t seq, size_t dim, size_t num_tiles, int round16,
                      void* stream);
@@ -205,6 +206,18 @@ int fv_vsa_attention(const void* q, const void* k, const void* v, int qkv_is_bf1
                      void* workspace, size_t workspace_bytes, uint32_t* selected_out, size_t bh,
                      size_t seq, size_t num_tiles, size_t topk, size_t dim, float scale, void* stream);
 
+/* fv_vsa_attention on operands a producer already wrote in tile-slot order (fv_qk_norm_rope_tiles,
+ * fv_split_heads_tiles): qt/kt/vt bf16 bits [bh, num_tiles*64, 128] with zero padding slots; gate
+ * and out stay in token order. The tile means read the tiles in place and the tile pass (three
+ * reads and writes of q/k/v) is skipped; the result is bit-identical to fv_vsa_attention on the
+ * token-ordered bf16 tensors. No counterpart in the reference, whose op always re-tiles
+ * (rt/vsa.rs:406-414). Needs only the first part of the workspace (fv_vsa_workspace_bytes is
+ * enough). */
+int fv_vsa_attention_tiled(const uint16_t* qt, const uint16_t* kt, const uint16_t* vt, const void* gate,
+                           int gate_is_bf16, const int32_t* slot_src, const int32_t* block_sizes, float* out,
+                           void* workspace, size_t workspace_bytes, uint32_t* selected_out, size_t bh,
+                           size_t seq, size_t num_tiles, size_t topk, size_t dim, float scale, void* stream);
+
 /* ---- producer / consumer either side of the SDPA call --------------------------------- */
 /* q/k RMSNorm across all heads (+ interleaved RoPE) of columns [col_off, col_off + heads*d) of
  * src [batch, seq, src_width], written as BHSD [batch, heads, seq, d].
@@ -220,10 +233,22 @@ int fv_qk_norm_rope_bhsd(const void* src, int src_is_bf16, const void* w, int w_
                          const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
                          size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
                          size_t col_off, float eps, void* stream);
+/* The same op writing VSA's tile-slot order: head planes are [padded, d] and token s lands in row
+ * token_slot[s] (fv_vsa_tile_plan; every value < padded, others are skipped). Padding rows are not
+ * written: zero `out` once, no call touches them afterwards. Feeds fv_vsa_attention_tiled. */
+int fv_qk_norm_rope_tiles(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
+                          const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
+                          size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
+                          size_t col_off, float eps, const uint32_t* token_slot, size_t padded,
+                          void* stream);
 /* rt/ops.rs:574-602 / kernels/core.cu:415-427 `split_heads_bhsd`: the value heads, a pure permute
  * of f32 or bf16 elements. */
 int fv_split_heads_bhsd(const void* src, void* out, int is_bf16, size_t batch, size_t seq, size_t heads,
                         size_t d, size_t src_width, size_t col_off, void* stream);
+/* fv_split_heads_bhsd into tile-slot order, as fv_qk_norm_rope_tiles. */
+int fv_split_heads_tiles(const void* src, void* out, int is_bf16, size_t batch, size_t seq, size_t heads,
+                         size_t d, size_t src_width, size_t col_off, const uint32_t* token_slot, size_t padded,
+                         void* stream);
 /* rt/ops.rs:604-620 / kernels/core.cu:429-443 `merge_heads`: BHSD -> [batch, seq, heads*d]. */
 int fv_merge_heads(const void* src, void* out, int is_bf16, size_t batch, size_t heads, size_t seq, size_t d,
                    void* stream);

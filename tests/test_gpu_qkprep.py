@@ -158,3 +158,40 @@ def test_producer_feeds_the_attention_kernel(fv, oracle):
     got = merged.float().cpu().numpy()
     assert got.shape == (batch, seq, heads * d)
     assert np.abs(got - want).max() <= 1e-2
+
+
+@pytest.mark.parametrize("grid", [(2, 3, 5), (5, 6, 9), (4, 4, 4)])
+@pytest.mark.parametrize("out16", [False, True])
+def test_tile_ordered_producers_are_the_bhsd_ones_permuted(fv, oracle, grid, out16):
+    """qk_norm_rope / split_heads writing VSA's tile-slot order: row token_slot[s] of the padded
+    plane holds exactly what row s of the BHSD plane holds, padding rows stay zero."""
+    import torch
+
+    ctx = fv.VsaCtx(grid, 0.8)
+    batch, heads, d = 2, 3, 128
+    announce(f"tile-ordered producers grid={grid} out16={out16}")
+    proj, w, cos, sin = _inputs(900 + ctx.seq, batch, ctx.seq, heads, d, 8, 2 * heads * d)
+    dt = torch.bfloat16 if out16 else torch.float32
+    tp = torch.from_numpy(proj).cuda().to(dt)
+    tw = torch.from_numpy(w).cuda().to(dt)
+    rope = (torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda())
+    col = 2 * heads * d
+    slot = torch.from_numpy(ctx.plan.token_slot.astype(np.int64)).cuda()
+    pad = torch.from_numpy(ctx.plan.slot_src < 0).cuda()
+    for r in (None, rope):
+        want = fv.qk_norm_rope_bhsd(tp, col, heads, tw, r, out_bf16=out16)
+        got = fv.qk_norm_rope_tiles(tp, col, heads, tw, ctx, r, out_bf16=out16)
+        torch.cuda.synchronize()
+        assert tuple(got.shape) == (batch, heads, ctx.padded, d) and got.dtype == want.dtype
+        assert torch.equal(got[:, :, slot], want)
+        assert not got[:, :, pad].any()
+    want = fv.split_heads_bhsd(tp, col, heads, d)
+    got = fv.split_heads_tiles(tp, col, heads, d, ctx)
+    torch.cuda.synchronize()
+    assert torch.equal(got[:, :, slot], want) and not got[:, :, pad].any()
+    # and against the oracle's own tile permute of the oracle's BHSD result (bf16 permute is exact)
+    if out16:
+        ref = oracle.split_heads_bhsd(oracle.quantize_bf16(proj), col, heads, d)
+        tiles = np.zeros((batch, heads, ctx.padded, d), np.float32)
+        tiles[:, :, ctx.plan.token_slot] = ref
+        assert np.array_equal(got.float().cpu().numpy(), tiles)

@@ -222,6 +222,38 @@ def test_whole_op_vs_host_oracle(fv, oracle, grid, in_bf16):
     assert torch.equal(a, bb)
 
 
+@pytest.mark.parametrize("grid", GRIDS + [(21, 30, 52)])
+def test_whole_op_on_tile_ordered_operands_is_bit_identical(fv, oracle, grid):
+    """fv_vsa_attention_tiled (q/k/v already in tile-slot order, as the tile-ordered producers write
+    them) == fv_vsa_attention on the token-ordered bf16 tensors: output and block lists bit for bit."""
+    import torch
+
+    announce(f"vsa tiled whole op grid={grid}")
+    ctx = fv.VsaCtx(grid, 0.8)
+    heads = 2
+    g = torch.Generator(device="cuda").manual_seed(71)
+    q, k, v, gate = (torch.randn((heads, ctx.seq, D), generator=g, device="cuda").to(torch.bfloat16) for _ in range(4))
+    scale = float(1.0 / np.sqrt(D))
+    slot = torch.from_numpy(ctx.plan.token_slot.astype(np.int64)).cuda()
+
+    def tiled(x):
+        t = torch.zeros((heads, ctx.padded, D), device="cuda", dtype=torch.bfloat16)
+        t[:, slot] = x
+        return t
+
+    for gt in (gate, None):
+        want, want_sel = fv.vsa_attention_device(q, k, v, gt, ctx, scale, return_selected=True)
+        got, sel = fv.vsa_attention_tiled(tiled(q), tiled(k), tiled(v), gt, ctx, scale, return_selected=True)
+        torch.cuda.synchronize()
+        assert torch.equal(sel, want_sel)
+        assert torch.equal(got, want)
+    # the stage entry reads tile-ordered input when slot_src is NULL
+    qc = fv.vsa_tile_mean(q, ctx)
+    qc_t = fv.vsa_tile_mean(tiled(q), ctx, tiled=True)
+    torch.cuda.synchronize()
+    assert torch.equal(qc, qc_t)
+
+
 def test_all_tiles_and_zero_gate_is_dense_attention(fv, oracle):
     """C/rt/vsa.rs:534-597 on the device: every tile selected + zero gate == dense SDPA."""
     import torch
