@@ -8,7 +8,7 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep) are for the
+Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache) are for the
 design notes; the driver's line is the default `self`.
 """
 import argparse
@@ -126,6 +126,76 @@ def bench_vsa(args):
                      "frac": round(fine_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::vsa_fine_kernel",
                      "avg_kernel_ms": round(stages["fine"], 4),
                      "banded_selection_tflops": round(flops / (stages["fine_banded_selection"] * 1e-3) / 1e12, 3)},
+    }
+    print(json.dumps(rec), flush=True)
+
+
+def bench_kvcache(args):
+    """Autoregressive Self-Forcing self-attention of one layer: 7 blocks of 3 latent frames (4680
+    tokens) written into a 21-frame KV cache and each block's queries attending the cache window in
+    place (Plan::kv_window). One step = the whole 7-block rollout of the layer: 7 cache writes + 7
+    dense calls of Sq = 4680 against Sk = 4680 ... 32760. The same with a contiguous copy of every
+    window first (what the reference's `narrow` does) is timed beside it."""
+    import torch
+
+    import fv_sdpa
+
+    lib = fv_sdpa.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    h, d, ft, fpb, frames = 12, 128, 1560, 3, 21
+    n, blocks = fpb * ft, frames // fpb
+    g = torch.Generator(device=dev).manual_seed(20243)
+    qs, ks, vs = ([torch.randn((1, h, n, d), generator=g, device=dev).to(torch.bfloat16) for _ in range(blocks)]
+                  for _ in range(3))
+    cache = fv_sdpa.CausalKvCache(fv_sdpa.KvSpec.global_window(ft, frames), 1)
+    plan = fv_sdpa.Plan.kv_window()
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = [torch.empty((h, n, d), device=dev, dtype=torch.bfloat16) for _ in range(blocks)]
+    scale = 1.0 / d ** 0.5
+
+    def rollout(copy_windows):
+        cache.reset()
+        for i in range(blocks):
+            kw, vw = cache.update(0, ks[i], vs[i], i * n)
+            if copy_windows:
+                kw, vw = kw.contiguous(), vw.contiguous()
+            sk = kw.shape[2]
+            rows = kw.stride(1) // d
+            rc = lib.fv_sdpa_dense_bf16_strided(qs[i].data_ptr(), kw.data_ptr(), vw.data_ptr(), outs[i].data_ptr(), 1,
+                                                h, n, sk, d, scale, 0, rows, rows, stream)
+            if rc != 0:
+                raise RuntimeError(lib.fv_sdpa_last_error().decode())
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    in_place = timed(lambda: rollout(False))
+    copied = timed(lambda: rollout(True))
+    # the plan entry once, to show it takes the same route
+    kw, vw = cache.update(0, ks[0], vs[0], 0)
+    before = fv_sdpa.rt_stats()
+    fv_sdpa.sdpa(qs[0], kw, vw, plan)
+    assert fv_sdpa.rt_stats()["fused"] == before["fused"] + 1
+    flops = sum(4.0 * h * n * (i + 1) * n * d for i in range(blocks))
+    tf = flops / (in_place * 1e-3) / 1e12
+    rec = {
+        "metric": "KV-window attention TFLOP/s (Self-Forcing rollout of one layer, cache read in place)",
+        "value": round(tf, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(in_place, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "7 blocks x 4680 queries against a 21-frame KV cache (Sk = 4680 ... 32760), H=12 d=128, "
+                               "cache write + attention per block", "flops_per_step": flops},
+        "ms_per_step_with_window_copies": round(copied, 4),
+        "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::flash_fwd_pp2<false, 128>"},
     }
     print(json.dumps(rec), flush=True)
 
@@ -264,7 +334,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep"])
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -288,6 +358,9 @@ def main():
         return
     if args.workload == "prep":
         bench_prep(args)
+        return
+    if args.workload == "kvcache":
+        bench_kvcache(args)
         return
     fv_sdpa.lib()
     dev = torch.device("cuda:0")

@@ -110,9 +110,9 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     int out_is_bf16 = p.out_is_bf16;
     asm volatile("" : "+s"(out_f32), "+s"(out_bf16), "+s"(out_is_bf16));
 
-    const uint16_t* Qh = p.q + ((size_t)bh * sq + q0) * kD;
-    const uint16_t* Kh = p.k + (size_t)bh * sk * kD;
-    const uint16_t* Vh = p.v + (size_t)bh * sk * kD;
+    const uint16_t* Qh = p.q + (size_t)bh * p.q_plane + (size_t)q0 * kD;
+    const uint16_t* Kh = p.k + (size_t)bh * p.k_plane;
+    const uint16_t* Vh = p.v + (size_t)bh * p.v_plane;
 
     const int nkt = (sk + kBN - 1) / kBN;
     // The key-tile walk of this query tile: up to three ascending tile ranges [a_i, a_i + n_i),

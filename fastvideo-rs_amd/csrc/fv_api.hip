@@ -55,6 +55,7 @@ enum { kMaskNone = 0, kMaskBlockCausal = 1, kMaskVdnWindow = 2 };
 
 struct MaskArgs {
     int mode = kMaskNone;
+    size_t q_rows = 0, k_rows = 0, v_rows = 0;   // rows per (batch, head) plane; 0 = contiguous (sq / sk)
     size_t block_tokens = 0, window = 0, sink = 0;                           // block-causal
     size_t video_start = 0, frame_tokens = 0, frames = 0, chunk = 0, radius = 0;   // VDN window
 };
@@ -65,6 +66,8 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
     if (!fv_sdpa_supported(1, bh, sq, sk, d)) return decline("sdpa: shape not taken by the fused kernel");
     if (!(scale > 0.0f) || !(scale < 3.0e38f)) return decline("sdpa: the fused kernel needs a finite scale > 0");
     if (!q || !k || !v || !out) return fv_invalid("sdpa: null operand");
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
+        return fv_invalid("sdpa: operands must be 16-byte aligned");
     fv::FlashParams p;
     p.q = q;
     p.k = k;
@@ -75,6 +78,15 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
     p.sq = (int)sq;
     p.sk = (int)sk;
     p.sl2 = scale * 1.4426950408889634f;
+    const size_t q_rows = m.q_rows ? m.q_rows : sq, k_rows = m.k_rows ? m.k_rows : sk,
+                 v_rows = m.v_rows ? m.v_rows : sk;
+    if (q_rows < sq || k_rows < sk || v_rows < sk) return fv_invalid("sdpa: plane rows below the sequence length");
+    const size_t plane_lim = (size_t)LONG_MAX / (d * (bh ? bh : 1));
+    if (q_rows > plane_lim || k_rows > plane_lim || v_rows > plane_lim)
+        return decline("sdpa: planes too large");
+    p.q_plane = (long)(q_rows * d);
+    p.k_plane = (long)(k_rows * d);
+    p.v_plane = (long)(v_rows * d);
     const size_t bm = (size_t)fv_internal_flash_block_m();
     p.nqt = (int)((sq + bm - 1) / bm);
     const size_t total = bh * (size_t)p.nqt;
@@ -136,6 +148,16 @@ int fv_sdpa_dense_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, 
                        int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                        void* stream) {
     return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, MaskArgs{}, stream);
+}
+
+int fv_sdpa_dense_bf16_strided(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
+                               int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
+                               size_t q_rows, size_t k_rows, size_t v_rows, void* stream) {
+    MaskArgs m;
+    m.q_rows = q_rows;
+    m.k_rows = k_rows;
+    m.v_rows = v_rows;
+    return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, m, stream);
 }
 
 int fv_sdpa_block_causal_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,

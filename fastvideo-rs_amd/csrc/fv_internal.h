@@ -23,6 +23,9 @@ struct FlashParams {
     int mask_mode;      // 0 none, 1 block-causal, 2 VDN window
     int ft, win, sink;  // block-causal: block tokens, window blocks, sink blocks; VDN window: ft = frame tokens
     int vs, ve, frames, chunk, radius;   // VDN window: video rows [vs, ve), frame count, chunk, radius
+    // elements between consecutive (batch, head) planes of q, k and v: s * d when contiguous, larger
+    // when the operand is a row window of a longer plane (a KV cache read in place)
+    long q_plane, k_plane, v_plane;
 };
 
 struct VsaFineParams {

@@ -1,0 +1,86 @@
+// The per-layer KV cache of causal (Self-Forcing) Wan generation and the arithmetic of its
+// pointers, mirroring crates/fastvideo-cudarc/src/wan/causal.rs:38-57 (`KvSpec`), 276-336
+// (`KvMove`, `KvSpec::plan`) and 341-723 (`CausalKvCache`, static mode): one persistent
+// [batch, heads, capacity, d] buffer pair per layer, written in place; the window the queries read
+// comes back as a row window of those buffers (no copy): the fused attention kernel reads a
+// (batch, head) plane at any plane stride.
+//
+// Built: absolute RoPE policy (keys arrive roped), rolling and global windows, the sink guard.
+// Not built: the relativistic and rebased-sink RoPE policies (they re-rope cached keys; the
+// constructor refuses them).
+#pragma once
+#include <mutex>
+#include <utility>
+
+#include "rt_sdpa.hpp"
+
+namespace fv::rt {
+
+// wan/causal.rs:38-57 (token geometry of one cache)
+struct KvSpec {
+    size_t frame_tokens = 0;    // tokens per latent frame
+    size_t capacity = 0;        // physical cache length in tokens
+    size_t sink = 0;            // tokens kept at the head when the cache rolls
+    size_t max_attention = 0;   // keys each query block reads, back from the end of the block
+    bool rolling = false;       // a full cache drops its oldest tokens after the sink instead of refusing
+};
+
+// wan/causal.rs:276-287
+struct KvMove {
+    size_t evicted = 0;                     // tokens dropped after the sink before writing
+    size_t local_start = 0, local_end = 0;  // where the block's K/V are written
+    size_t window_start = 0;                // the queries read [window_start, local_end)
+};
+
+// wan/causal.rs:289-336 `KvSpec::plan`: the pointer arithmetic for n new tokens at current_start
+// from the cache state (global_end, local_end_prev).
+Result<KvMove> kv_plan(const KvSpec& spec, size_t global_end, size_t local_end_prev, size_t current_start,
+                       size_t n);
+
+// wan/causal.rs:199-248 on device buffers [bh, rows, d] of f32 or bf16 elements:
+// dst[:, dst_off .. dst_off + len] = src[:, src_off .. src_off + len] ...
+int kv_copy_tokens(void* dst, size_t dst_rows, size_t dst_off, const void* src, size_t src_rows, size_t src_off,
+                   size_t len, size_t bh, size_t d, DType dtype, hipStream_t st);
+// ... and tokens [from, from + len) of t moved down to [to, to + len), to < from, in chunks no longer
+// than the shift so that no launch reads what it writes.
+int kv_shift_tokens_down(void* t, size_t rows, size_t from, size_t to, size_t len, size_t bh, size_t d,
+                         DType dtype, hipStream_t st);
+
+struct KvPointers {
+    size_t global_end = 0, local_end = 0;
+};
+
+// wan/causal.rs:341-723, `new_static` mode.
+class CausalKvCache {
+  public:
+    CausalKvCache(KvSpec spec, size_t num_layers);
+    ~CausalKvCache();
+    CausalKvCache(const CausalKvCache&) = delete;
+    CausalKvCache& operator=(const CausalKvCache&) = delete;
+
+    // Writes one block's k / v ([b, h, n, d], contiguous, same dtype, RoPE applied) for `layer` at
+    // token `current_start`; returns the K / V windows its queries attend to: borrowed row windows
+    // [b, h, len, d] of the layer's buffers (plane_rows = capacity), valid until the next write.
+    Result<std::pair<Tensor, Tensor>> update(size_t layer, const Tensor& k, const Tensor& v, size_t current_start,
+                                             hipStream_t st);
+    void reset();                         // a new rollout: pointers to zero, buffers (addresses) kept
+    void set_sink_guard(bool on) { sink_guard_ = on; }
+    bool sink_guard() const { return sink_guard_; }
+    std::vector<KvPointers> pointers() const;
+    size_t bytes() const;
+    const KvSpec spec;
+
+  private:
+    struct Layer {
+        void* k = nullptr;
+        void* v = nullptr;
+        size_t b = 0, h = 0, cap = 0, d = 0, dv = 0;
+        DType kd = DType::F32, vd = DType::F32;
+        size_t global_end = 0, local_end = 0;
+    };
+    mutable std::mutex mu_;
+    std::vector<Layer> layers_;
+    bool sink_guard_ = false;
+};
+
+}  // namespace fv::rt

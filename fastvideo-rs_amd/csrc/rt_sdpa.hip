@@ -9,6 +9,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <tuple>
 
 #include "../../include/fv_sdpa_hip.h"
 #include "fv_common.h"
@@ -184,6 +185,20 @@ float default_scale(std::optional<float> scale, size_t d) {
     return scale ? *scale : 1.0f / sqrtf((float)d);
 }
 
+// A contiguous copy of a row window (what the reference's `narrow` always makes).
+Result<Tensor> compact(const Tensor& x, hipStream_t st) {
+    auto r = Tensor::alloc(x.shape, x.dtype, st);
+    if (!is_ok(r)) return r;
+    Tensor t = std::move(std::get<Tensor>(r));
+    const size_t row = x.shape[3] * elem_size(x.dtype), planes = x.shape[0] * x.shape[1];
+    if (planes && x.shape[2] && row) {
+        const hipError_t e = hipMemcpy2DAsync(t.data, x.shape[2] * row, x.data, x.plane_rows * row, x.shape[2] * row,
+                                              planes, hipMemcpyDeviceToDevice, st);
+        if (e != hipSuccess) return msg(std::string("sdpa: compacting a row window: ") + hipGetErrorString(e));
+    }
+    return std::move(t);
+}
+
 // One fused launch (dense, block-causal or VDN window); nullopt = the kernel declined.
 Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tensor& v,
                                     std::optional<float> scale, bool out_bf16,
@@ -213,6 +228,9 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
         rc = fv_sdpa_vdn_window_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
                                      window->video_start, window->frame_tokens, window->frames, window->chunk,
                                      window->radius, st);
+    else if (q.strided() || k.strided() || v.strided())
+        rc = fv_sdpa_dense_bf16_strided(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
+                                        q.plane_rows, k.plane_rows, v.plane_rows, st);
     else
         rc = fv_sdpa_dense_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc, st);
     if (rc == FV_DECLINED) return std::optional<Tensor>{};
@@ -335,6 +353,7 @@ Tensor& Tensor::operator=(Tensor&& o) noexcept {
         shape = std::move(o.shape);
         dtype = o.dtype;
         data = o.data;
+        plane_rows = o.plane_rows;
         owned_ = o.owned_;
         stream_ = o.stream_;
         o.data = nullptr;
@@ -350,6 +369,11 @@ Tensor Tensor::borrowed(void* data, std::vector<size_t> shape, DType dtype) {
     t.data = data;
     t.shape = std::move(shape);
     t.dtype = dtype;
+    return t;
+}
+Tensor Tensor::window(void* data, std::vector<size_t> shape, DType dtype, size_t plane_rows) {
+    Tensor t = borrowed(data, std::move(shape), dtype);
+    t.plane_rows = t.shape.size() == 4 && plane_rows != t.shape[2] ? plane_rows : 0;
     return t;
 }
 Result<Tensor> Tensor::alloc(std::vector<size_t> shape, DType dtype, hipStream_t stream) {
@@ -553,6 +577,29 @@ Result<Tensor> sdpa_composed(const Tensor& q, const Tensor& k, const Tensor& v, 
 
 Result<Tensor> sdpa(const Tensor& q, const Tensor& k, const Tensor& v, const Plan& plan, hipStream_t st) {
     if (q.rank() != 4 || k.rank() != 4 || v.rank() != 4) return msg("sdpa expects BHSD");
+    if (q.strided() || k.strided() || v.strided()) {
+        // Row windows of longer planes (a KV cache read in place). The fused dense kernel takes bf16
+        // windows as they are; every other path gets contiguous copies.
+        const bool dense_like = (plan.kind == Plan::Kind::Dense && !plan.mask) ||
+                                (plan.kind == Plan::Kind::KvWindow && plan.kv_flash.value_or(causal_flash_enabled()));
+        const bool all16 = q.dtype == DType::Bf16 && k.dtype == DType::Bf16 && v.dtype == DType::Bf16;
+        if (dense_like && all16 && backend() == Backend::Dense) {
+            auto r = fused(q, k, v, plan.scale, bf16_activations(), nullptr, st);
+            if (!is_ok(r)) return std::get<TensorError>(r);
+            auto& o = std::get<std::optional<Tensor>>(r);
+            if (o) return std::move(*o);
+        }
+        Tensor cq, ck, cv;
+        const Tensor *pq = &q, *pk = &k, *pv = &v;
+        for (auto [src, tmp, dst] : {std::tuple{&q, &cq, &pq}, std::tuple{&k, &ck, &pk}, std::tuple{&v, &cv, &pv}}) {
+            if (!src->strided()) continue;
+            auto r = compact(*src, st);
+            if (!is_ok(r)) return std::get<TensorError>(r);
+            *tmp = std::move(std::get<Tensor>(r));
+            *dst = tmp;
+        }
+        return sdpa(*pq, *pk, *pv, plan, st);
+    }
     switch (plan.kind) {
         case Plan::Kind::Dense:
             // fp8_first marks H3's FP8 QK^T attempt (rt/sdpa.rs:148-158); this library is bf16 only
@@ -581,8 +628,11 @@ int fv_rt_sdpa(const fv_tensor* q, const fv_tensor* k, const fv_tensor* v, const
     if (!q || !k || !v || !plan || !out) return fv_invalid("fv_rt_sdpa: null argument");
     auto wrap = [](const fv_tensor* t) {
         std::vector<size_t> shape(t->shape, t->shape + (t->rank < 0 ? 0 : (t->rank > 8 ? 8 : t->rank)));
-        return Tensor::borrowed(t->data, std::move(shape), t->dtype ? DType::Bf16 : DType::F32);
+        return Tensor::window(t->data, std::move(shape), t->dtype ? DType::Bf16 : DType::F32, t->plane_rows);
     };
+    for (const fv_tensor* t : {q, k, v})
+        if (t->plane_rows != 0 && (t->rank != 4 || t->plane_rows < t->shape[2]))
+            return fv_invalid("fv_rt_sdpa: plane_rows needs a rank-4 operand and plane_rows >= shape[2]");
     const Tensor tq = wrap(q), tk = wrap(k), tv = wrap(v);
     Tensor tmask;
     if (plan->mask) tmask = wrap(plan->mask);
@@ -615,6 +665,7 @@ int fv_rt_sdpa(const fv_tensor* q, const fv_tensor* k, const fv_tensor* v, const
     out->rank = (int)t.rank();
     for (size_t i = 0; i < t.rank() && i < 8; i++) out->shape[i] = t.shape[i];
     out->dtype = t.dtype == DType::Bf16 ? 1 : 0;
+    out->plane_rows = 0;
     out->data = t.release();
     return FV_OK;
 }

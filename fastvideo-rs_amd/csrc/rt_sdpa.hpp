@@ -43,9 +43,14 @@ class Tensor {
     ~Tensor();
 
     static Tensor borrowed(void* data, std::vector<size_t> shape, DType dtype);
+    // A borrowed rank-4 row window: [b, h, s, d] whose (batch, head) planes sit plane_rows * d
+    // elements apart in the underlying buffer (plane_rows >= s; 0 = contiguous). What `narrow(2, ..)`
+    // of a longer BHSD tensor is without the copy (rt/tensor.rs:825-870 copies).
+    static Tensor window(void* data, std::vector<size_t> shape, DType dtype, size_t plane_rows);
     static Result<Tensor> alloc(std::vector<size_t> shape, DType dtype, hipStream_t stream);
 
     size_t rank() const { return shape.size(); }
+    bool strided() const { return plane_rows != 0 && shape.size() == 4 && plane_rows != shape[2]; }
     size_t numel() const;
     // Gives up ownership of the buffer (the caller frees it with hipFree).
     void* release();
@@ -53,6 +58,7 @@ class Tensor {
     std::vector<size_t> shape;
     DType dtype = DType::F32;
     void* data = nullptr;
+    size_t plane_rows = 0;   // rows per (batch, head) plane of the storage; 0 = shape[2]
 
   private:
     bool owned_ = false;

@@ -7,3 +7,4 @@ from .ops import *  # noqa: F401,F403
 from .vsa import *  # noqa: F401,F403
 from .sdpa import *  # noqa: F401,F403
 from .prep import *  # noqa: F401,F403
+from .kv_cache import *  # noqa: F401,F403

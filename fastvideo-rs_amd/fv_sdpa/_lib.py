@@ -22,6 +22,18 @@ SIGNATURES = {
     "fv_sdpa_arch": (C.c_char_p, []),
     "fv_sdpa_supported": (C.c_int, [_sz, _sz, _sz, _sz, _sz]),
     "fv_sdpa_dense_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float, _vp]),
+    "fv_sdpa_dense_bf16_strided": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float, _sz, _sz, _sz,
+                                             _vp]),
+    "fv_kv_plan": (C.c_int, [_sz, _sz, _sz, _sz, C.c_int, _sz, _sz, _sz, _sz, _vp]),
+    "fv_kv_copy_tokens": (C.c_int, [_vp, _sz, _sz, _vp, _sz, _sz, _sz, _sz, _sz, C.c_int, _vp]),
+    "fv_kv_shift_tokens_down": (C.c_int, [_vp, _sz, _sz, _sz, _sz, _sz, _sz, C.c_int, _vp]),
+    "fv_kv_cache_new": (_vp, [_sz, _sz, _sz, _sz, C.c_int, _sz]),
+    "fv_kv_cache_free": (None, [_vp]),
+    "fv_kv_cache_reset": (None, [_vp]),
+    "fv_kv_cache_set_sink_guard": (None, [_vp, C.c_int]),
+    "fv_kv_cache_pointers": (C.c_int, [_vp, _sz, _vp]),
+    "fv_kv_cache_bytes": (_sz, [_vp]),
+    "fv_kv_cache_update": (C.c_int, [_vp, _sz, _vp, _vp, _sz, _vp, _vp, _vp]),
     "fv_sdpa_block_causal_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float,
                                             _sz, _sz, _sz, _vp]),
     "fv_cast_f32_bf16": (C.c_int, [_vp, _vp, _sz, _vp]),

@@ -9,7 +9,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["sdpa_dense_bf16", "sdpa_block_causal_bf16", "sdpa_vdn_window_bf16", "cast_f32_bf16", "cast_bf16_f32", "sdpa_supported"]
+__all__ = ["sdpa_dense_bf16", "sdpa_dense_bf16_windows", "sdpa_block_causal_bf16", "sdpa_vdn_window_bf16", "cast_f32_bf16", "cast_bf16_f32", "sdpa_supported"]
 
 
 def _stream():
@@ -42,6 +42,33 @@ def sdpa_dense_bf16(q, k, v, scale=None, out_bf16=False):
     out = torch.empty((bh, sq, d), device=q.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
     _lib.check(_lib.lib().fv_sdpa_dense_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                              int(out_bf16), bh, sq, sk, d, scale, _stream()))
+    return out
+
+
+def _plane_rows(t, name):
+    """Rows per plane of a [bh, s, d] bf16 tensor that is contiguous or a row window
+    (`base[:, a:b]`) of a contiguous [bh, rows, d] tensor."""
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.bfloat16 and t.dim() == 3):
+        raise ValueError(f"{name}: want a [bh, s, d] CUDA bf16 tensor")
+    bh, s, d = t.shape
+    sb, ss, sd = t.stride()
+    if sd != 1 or ss != d or (bh > 1 and (sb % d or sb < s * d)):
+        raise ValueError(f"{name}: want contiguous rows and one plane stride (a row window of a [bh, rows, d] tensor)")
+    return sb // d if bh > 1 else s
+
+
+def sdpa_dense_bf16_windows(q, k, v, scale=None, out_bf16=False):
+    """`sdpa_dense_bf16` on row windows of longer planes (`cache[:, start:end]`), read in place."""
+    rows = [_plane_rows(t, n) for t, n in ((q, "q"), (k, "k"), (v, "v"))]
+    bh, sq, d = q.shape
+    if k.shape != v.shape or k.shape[0] != bh or k.shape[2] != d:
+        raise ValueError(f"k/v {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
+    sk = k.shape[1]
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    out = torch.empty((bh, sq, d), device=q.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    _lib.check(_lib.lib().fv_sdpa_dense_bf16_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                                     int(out_bf16), bh, sq, sk, d, scale, rows[0], rows[1], rows[2],
+                                                     _stream()))
     return out
 
 

@@ -18,7 +18,8 @@ class TensorError(RuntimeError):
 
 
 class _FvTensor(C.Structure):
-    _fields_ = [("data", C.c_void_p), ("dtype", C.c_int), ("rank", C.c_int), ("shape", C.c_size_t * 8)]
+    _fields_ = [("data", C.c_void_p), ("dtype", C.c_int), ("rank", C.c_int), ("shape", C.c_size_t * 8),
+                ("plane_rows", C.c_size_t)]
 
 
 class _FvPlan(C.Structure):
@@ -110,8 +111,25 @@ class Plan:
         return Plan(Plan.KV_WINDOW, kv_flash=bool(flash))
 
 
+def _window_rows(t):
+    """plane_rows of a BHSD tensor that is a row window (`base[:, :, a:b]`) of a contiguous
+    [b, h, rows, d] tensor, else None."""
+    if t.dim() != 4:
+        return None
+    b, h, s, d = t.shape
+    sb, sh, ss, sd = t.stride()
+    if sd != 1 or ss != d or sh % d or sh < s * d or (b > 1 and sb != h * sh):
+        return None
+    return sh // d
+
+
 def _desc(t, name):
-    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.is_contiguous()):
+    rows = 0
+    if isinstance(t, torch.Tensor) and t.is_cuda and not t.is_contiguous():
+        rows = _window_rows(t) or 0
+        if not rows:
+            raise ValueError(f"{name}: want a contiguous CUDA tensor or a row window of a BHSD one")
+    elif not (isinstance(t, torch.Tensor) and t.is_cuda):
         raise ValueError(f"{name}: want a contiguous CUDA tensor")
     if t.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError(f"{name}: want f32 or bf16")
@@ -119,6 +137,7 @@ def _desc(t, name):
         raise ValueError(f"{name}: rank > 8")
     d = _FvTensor()
     d.data, d.dtype, d.rank = t.data_ptr(), int(t.dtype == torch.bfloat16), t.dim()
+    d.plane_rows = rows
     for i, s in enumerate(t.shape):
         d.shape[i] = s
     return d

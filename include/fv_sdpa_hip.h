@@ -45,6 +45,14 @@ int fv_sdpa_dense_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, 
                        int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                        void* stream);
 
+/* fv_sdpa_dense_bf16 on row windows of longer planes: the (batch, head) planes of q / k / v sit
+ * q_rows / k_rows / v_rows rows of d elements apart (0 = contiguous: sq / sk). The KV-cache window of
+ * autoregressive generation (wan/causal.rs:700-704, wan/transformer.rs:292-294) is read in place
+ * instead of being copied out by `narrow`. out is contiguous [bh, sq, d]. */
+int fv_sdpa_dense_bf16_strided(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
+                               int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
+                               size_t q_rows, size_t k_rows, size_t v_rows, void* stream);
+
 /* rt/attn.rs:652-730 `device_mma_sdpa_causal` + kernels/attn2.cu:626-642
  * `flash_mma_fwd2_causal_d128`: the same under BlockCausal{block_tokens,
  * window, sink} (rt/attn.rs:441-453): query i sees key j iff
@@ -87,6 +95,9 @@ typedef struct fv_tensor {
     int dtype;         /* 0 = f32, 1 = bf16 bits (rt/tensor.rs:28-32) */
     int rank;
     size_t shape[8];
+    size_t plane_rows; /* 0: contiguous. Else (rank 4 only) the [b,h] planes of `data` sit plane_rows * d
+                          elements apart, plane_rows >= shape[2]: a row window of a longer BHSD buffer
+                          (a KV cache read in place), what rt/tensor.rs:825 `narrow(2, ..)` copies out */
 } fv_tensor;
 
 enum {
@@ -135,6 +146,42 @@ int fv_rt_dense_route(const size_t* q_shape, const size_t* k_shape, const size_t
 /* rt/stats.rs:27-72 analogue: {fused dense launches, block-causal launches, composed launches,
  * cast launches, dense masks materialised} since the library was loaded. */
 void fv_rt_stats(uint64_t out5[5]);
+
+/* ---- the KV cache of causal (Self-Forcing) Wan generation (wan/causal.rs) ----------------------
+ * wan/causal.rs:289-336 `KvSpec::plan`: where n new tokens at current_start go in a cache in state
+ * (global_end, local_end_prev). move_out = {evicted, local_start, local_end, window_start}. Host only;
+ * a negative return carries the reference's message in fv_sdpa_last_error(). */
+int fv_kv_plan(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
+               size_t global_end, size_t local_end_prev, size_t current_start, size_t n, size_t move_out[4]);
+/* wan/causal.rs:199-232 `copy_tokens` on device buffers [bh, rows, d] (f32 or bf16 elements, rows of a
+ * 16-byte multiple): dst[:, dst_off .. dst_off + len] = src[:, src_off .. src_off + len]. */
+int fv_kv_copy_tokens(void* dst, size_t dst_rows, size_t dst_off, const void* src, size_t src_rows, size_t src_off,
+                      size_t len, size_t bh, size_t d, int is_bf16, void* stream);
+/* wan/causal.rs:234-248 `shift_tokens_down`: tokens [from, from + len) of t [bh, rows, d] move down to
+ * [to, to + len), to < from, in launches no longer than the shift (none reads what it writes). */
+int fv_kv_shift_tokens_down(void* t, size_t rows, size_t from, size_t to, size_t len, size_t bh, size_t d,
+                            int is_bf16, void* stream);
+/* wan/causal.rs:341-723 `CausalKvCache::new_static`: one persistent [b, h, capacity, d] K / V pair per
+ * layer (allocated with hipMalloc at the layer's first write, kept by fv_kv_cache_reset). The RoPE
+ * policy is the absolute one (keys arrive roped); the relativistic and rebased-sink policies are not
+ * built. fv_kv_cache_update = `update`: rolls (wan/causal.rs:678-690), writes the block's k / v
+ * [b, h, n, d] at current_start and returns the windows the block's queries read as row windows of
+ * the layer's buffers (plane_rows = capacity; valid until the layer's next update): pass them to
+ * fv_rt_sdpa with FV_PLAN_KV_WINDOW (or fv_sdpa_dense_bf16_strided). Errors carry the reference's
+ * messages. One cache is driven from one thread at a time per layer (a mutex serialises the host
+ * bookkeeping); the device work is ordered on `stream`. */
+typedef struct fv_kv_cache fv_kv_cache;
+fv_kv_cache* fv_kv_cache_new(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
+                             size_t layers);
+void fv_kv_cache_free(fv_kv_cache* c);
+void fv_kv_cache_reset(fv_kv_cache* c);
+/* wan/causal.rs:396-418 `set_sink_guard`: a write that re-runs cached frames leaves the sink slots. */
+void fv_kv_cache_set_sink_guard(fv_kv_cache* c, int on);
+/* out2 = {global_end, local_end} of a layer (wan/causal.rs:431-445 `pointers`). */
+int fv_kv_cache_pointers(const fv_kv_cache* c, size_t layer, size_t out2[2]);
+size_t fv_kv_cache_bytes(const fv_kv_cache* c);
+int fv_kv_cache_update(fv_kv_cache* c, size_t layer, const fv_tensor* k, const fv_tensor* v, size_t current_start,
+                       fv_tensor* k_window, fv_tensor* v_window, void* stream);
 
 /* ---- Video Sparse Attention (rt/vsa.rs, rt/ops.rs:811-1619) --------------------------
  * Geometry: 64-token cubes (4x4x4 in t,h,w), TilePlan arrays as rt/vsa.rs:42-109:

@@ -5,3 +5,4 @@ package. It is the parity checker and the timed CPU baseline, never the
 product path.
 """
 from .binding import *  # noqa: F401,F403
+from .kv_cache import *  # noqa: F401,F403,E402

@@ -1,0 +1,223 @@
+"""The causal-Wan KV cache on the device, through the C ABI: token copies and the in-place roll are
+bit-exact against numpy; a cache driven block by block holds, after every write, exactly the window
+the oracle's restatement of the reference holds (crates/fastvideo-cudarc/src/wan/causal.rs:540-706);
+the fused kernel reading that window in place is bit-identical to the same kernel on a contiguous
+copy; and block by block through the cache equals the whole clip under the block-causal mask
+(the reference's own invariant, causal.rs:916-1000) within the kernel tolerance.
+"""
+import numpy as np
+import pytest
+
+from util import announce, assert_parity, qkv, to_dev_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fv():
+    import torch
+
+    assert torch.cuda.is_available()
+    import fv_sdpa
+
+    fv_sdpa.lib()
+    return fv_sdpa
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_copy_and_shift_tokens_bit_exact(fv, bf16):
+    import torch
+
+    announce(f"kv copy/shift bf16={bf16}")
+    dt = torch.bfloat16 if bf16 else torch.float32
+    bh, rows, d = 5, 37, 64
+    g = torch.Generator(device="cuda").manual_seed(3)
+    dst = torch.randn((bh, rows, d), generator=g, device="cuda").to(dt)
+    src = torch.randn((bh, 11, d), generator=g, device="cuda").to(dt)
+    want = dst.clone()
+    want[:, 20:27] = src[:, 3:10]
+    fv.kv_copy_tokens(dst, 20, src, 3, 7)
+    torch.cuda.synchronize()
+    assert torch.equal(dst, want)
+    # a shift shorter than the moved range: source and destination overlap, chunks must not
+    for frm, to, n in ((9, 4, 25), (30, 0, 7), (5, 4, 32), (12, 12, 3)):
+        t = torch.randn((bh, rows, d), generator=g, device="cuda").to(dt)
+        want = t.clone()
+        want[:, to:to + n] = t[:, frm:frm + n].clone()
+        fv.kv_shift_tokens_down(t, frm, to, n)
+        torch.cuda.synchronize()
+        assert torch.equal(t, want), (frm, to, n)
+    with pytest.raises(fv.FvError):
+        fv.kv_copy_tokens(dst, 35, src, 0, 7)          # past the destination
+    with pytest.raises(fv.FvError):
+        fv.kv_shift_tokens_down(dst, 3, 9, 4)          # tokens only move down
+
+
+@pytest.mark.parametrize("d", [128, 64])
+def test_row_windows_are_read_in_place_bit_identically(fv, d):
+    import torch
+
+    announce(f"strided dense d={d}")
+    bh, rows_q, rows_kv = 3, 400, 1000
+    g = torch.Generator(device="cuda").manual_seed(5)
+    Q = torch.randn((bh, rows_q, d), generator=g, device="cuda").to(torch.bfloat16)
+    K = torch.randn((bh, rows_kv, d), generator=g, device="cuda").to(torch.bfloat16)
+    V = torch.randn((bh, rows_kv, d), generator=g, device="cuda").to(torch.bfloat16)
+    for (q0, q1), (k0, k1) in (((0, 400), (0, 1000)), ((17, 300), (130, 899)), ((399, 400), (0, 1)), ((5, 261), (936, 1000))):
+        q, k, v = Q[:, q0:q1], K[:, k0:k1], V[:, k0:k1]
+        want = fv.sdpa_dense_bf16(q.contiguous(), k.contiguous(), v.contiguous())
+        got = fv.sdpa_dense_bf16_windows(q, k, v)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), ((q0, q1), (k0, k1))
+    with pytest.raises(ValueError):
+        fv.sdpa_dense_bf16_windows(Q[:, ::2], K, V)
+
+
+def _blocks(seed, b, h, n, d, count):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return [(rng.standard_normal((b, h, n, d)).astype(np.float32), rng.standard_normal((b, h, n, d)).astype(np.float32))
+            for _ in range(count)]
+
+
+CACHES = [
+    # frame_tokens, capacity frames, sink frames, rolling, block frames, blocks
+    (6, 7, 0, False, 2, 3),      # global window, appends only
+    (6, 6, 1, True, 3, 5),       # the reference's rolling example geometry (causal.rs:888-910)
+    (5, 8, 2, True, 3, 6),       # capacity not a multiple of the block: partial evictions
+    (4, 5, 0, True, 2, 6),       # no sink
+]
+
+
+@pytest.mark.parametrize("case", CACHES)
+@pytest.mark.parametrize("bf16", [True, False])
+def test_cache_windows_equal_the_oracles(fv, oracle, case, bf16):
+    import torch
+
+    ft, cap_f, sink_f, rolling, blk_f, count = case
+    announce(f"kv cache {case} bf16={bf16}")
+    b, h, d, layers = 2, 3, 64, 2
+    n = blk_f * ft
+    spec = fv.KvSpec(ft, cap_f * ft, sink_f * ft, cap_f * ft, rolling)
+    ospec = oracle.KvSpecO(ft, cap_f * ft, sink_f * ft, cap_f * ft, rolling)
+    cache, ocache = fv.CausalKvCache(spec, layers), oracle.CausalKvCacheO(ospec, layers)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    rnd = (lambda x: oracle.quantize_bf16(x)) if bf16 else (lambda x: x)
+    dev = lambda x: torch.from_numpy(x).cuda().to(dt)  # noqa: E731
+    for layer in range(layers):
+        for i, (k, v) in enumerate(_blocks(100 * layer + ft, b, h, n, d, count)):
+            k, v = rnd(k), rnd(v)
+            for step in range(2):    # every block runs twice: an append, then an overwrite in place
+                kk = k if step == 0 else rnd(k * 0.5)
+                want_k, want_v = ocache.update(layer, kk, v, i * n)
+                kw, vw = cache.update(layer, dev(kk), dev(v), i * n)
+                torch.cuda.synchronize()
+                assert tuple(kw.shape) == want_k.shape and kw.dtype == dt
+                assert np.array_equal(kw.float().cpu().numpy(), want_k), (layer, i, step)
+                assert np.array_equal(vw.float().cpu().numpy(), want_v), (layer, i, step)
+                o = ocache.layers[layer]
+                assert cache.pointers(layer) == (o.global_end, o.local_end)
+    assert cache.bytes() == layers * 2 * b * h * max(cap_f * ft, n) * d * (2 if bf16 else 4)
+    # a new rollout keeps the buffers and starts from empty pointers
+    cache.reset()
+    ocache.reset()
+    assert cache.pointers(0) == (0, 0)
+    k, v = _blocks(7, b, h, n, d, 1)[0]
+    kw, _ = cache.update(0, dev(rnd(k)), dev(rnd(v)), 0)
+    torch.cuda.synchronize()
+    assert np.array_equal(kw.float().cpu().numpy(), ocache.update(0, rnd(k), rnd(v), 0)[0])
+
+
+def test_cache_errors_and_sink_guard(fv, oracle):
+    import torch
+
+    announce("kv cache errors / sink guard")
+    b, h, d, ft = 1, 2, 64, 4
+    dev = lambda x: torch.from_numpy(x).cuda().to(torch.bfloat16)  # noqa: E731
+    glob = fv.CausalKvCache(fv.KvSpec.global_window(ft, 3), 1)
+    blk = _blocks(1, b, h, 2 * ft, d, 1)[0]
+    glob.update(0, dev(blk[0]), dev(blk[1]), 0)
+    with pytest.raises(fv.TensorError, match="local_attn_size=-1 keeps a 3-frame KV window"):
+        glob.update(0, dev(blk[0]), dev(blk[1]), 2 * ft)
+    with pytest.raises(fv.TensorError, match="no layer 4"):
+        glob.update(4, dev(blk[0]), dev(blk[1]), 0)
+    with pytest.raises(fv.TensorError, match="do not fit these keys"):
+        glob.update(0, dev(blk[0][:, :1]), dev(blk[1][:, :1]), 0)
+    # sink guard (causal.rs:396-418): a recompute of cached frames leaves the sink slots as they are
+    spec, ospec = fv.KvSpec(ft, 6 * ft, ft, 6 * ft, True), oracle.KvSpecO(ft, 6 * ft, ft, 6 * ft, True)
+    cache, ocache = fv.CausalKvCache(spec, 1), oracle.CausalKvCacheO(ospec, 1)
+    q16 = oracle.quantize_bf16
+    for i, (k, v) in enumerate(_blocks(2, b, h, 3 * ft, d, 2)):
+        cache.update(0, dev(k), dev(v), i * 3 * ft)
+        ocache.update(0, q16(k), q16(v), i * 3 * ft)
+    cache.set_sink_guard(True)
+    ocache.sink_guard = True
+    k, v = _blocks(3, b, h, 6 * ft, d, 1)[0]
+    # frames [0, 6) again from current_start 0 is not a recompute; from a later start it is
+    for start, kk, vv in ((0, k, v), (3 * ft, k[:, :, :3 * ft], v[:, :, :3 * ft])):
+        want_k, want_v = ocache.update(0, q16(kk), q16(vv), start)
+        kw, vw = cache.update(0, dev(kk), dev(vv), start)
+        torch.cuda.synchronize()
+        assert np.array_equal(kw.float().cpu().numpy(), want_k) and np.array_equal(vw.float().cpu().numpy(), want_v)
+
+
+@pytest.mark.parametrize("act16", [True, False])
+def test_kv_window_plan_reads_the_cache_in_place(fv, oracle, act16):
+    """sdpa(q, kw, vw, Plan::kv_window()) (wan/transformer.rs:292-294) on the windows of a rolling
+    cache: bit-identical to the fused kernel on contiguous copies, and within tolerance of the
+    fp32 oracle on the window."""
+    import torch
+
+    b, h, d, ft = 1, 3, 128, 40
+    n, layers = 3 * ft, 1
+    announce(f"kv window plan act16={act16}")
+    spec = fv.KvSpec.rolling_window(ft, 9, 1)
+    cache = fv.CausalKvCache(spec, layers)
+    ocache = oracle.CausalKvCacheO(oracle.KvSpecO(ft, 9 * ft, ft, 9 * ft, True), layers)
+    with fv.with_bf16_act(act16):
+        for i in range(5):
+            q, k, v = (x.reshape(b, h, n, d) for x in qkv(500 + i, b * h, n, n, d))
+            kw, vw = cache.update(0, to_dev_bf16(k), to_dev_bf16(v), i * n)
+            want_k, want_v = ocache.update(0, oracle.quantize_bf16(k), oracle.quantize_bf16(v), i * n)
+            assert not kw.is_contiguous() or kw.shape[2] == spec.capacity
+            before = fv.rt_stats()
+            got = fv.sdpa(to_dev_bf16(q), kw, vw, fv.Plan.kv_window())
+            after = fv.rt_stats()
+            assert after["fused"] == before["fused"] + 1 and after["composed"] == before["composed"]
+            assert got.dtype == (torch.bfloat16 if act16 else torch.float32)
+            direct = fv.sdpa_dense_bf16(to_dev_bf16(q).reshape(b * h, n, d), kw.reshape(b * h, -1, d).contiguous(),
+                                        vw.reshape(b * h, -1, d).contiguous(), out_bf16=act16)
+            torch.cuda.synchronize()
+            assert torch.equal(got.reshape(b * h, n, d), direct)
+            sk = want_k.shape[2]
+            want = oracle.sdpa_composed(q.reshape(b * h, n, d), want_k.reshape(b * h, sk, d), want_v.reshape(b * h, sk, d))
+            assert_parity(got.float().cpu().numpy().reshape(b * h, n, d), want, f"kv_window_block{i}",
+                          max_abs=2e-2 if act16 else 1e-2)
+        # the composed route (FASTVIDEO_WAN_CAUSAL_FLASH=0) takes contiguous copies of the windows
+        got_c = fv.sdpa(to_dev_bf16(q), kw, vw, fv.Plan.kv_window_with(False))
+        torch.cuda.synchronize()
+        assert_parity(got_c.float().cpu().numpy().reshape(b * h, n, d), want, "kv_window_composed",
+                      max_abs=2e-2 if act16 else 1e-5)
+
+
+def test_cached_blocks_equal_the_masked_whole_clip(fv, oracle):
+    """causal.rs:916-1000: block by block through a global-window cache is the whole clip under the
+    block-causal mask: every query meets the same keys."""
+    import torch
+
+    bh, d, ft, fpb, frames = 4, 128, 90, 3, 9
+    n, s = fpb * ft, frames * ft
+    announce("kv cache blocks == block-causal whole clip")
+    q, k, v = qkv(77, bh, s, s, d)
+    whole = fv.sdpa_block_causal_bf16(to_dev_bf16(q), to_dev_bf16(k), to_dev_bf16(v), n, 0, 0)
+    cache = fv.CausalKvCache(fv.KvSpec.global_window(ft, frames), 1)
+    r4 = lambda x, a, bnd: to_dev_bf16(x[:, a:bnd]).reshape(1, bh, bnd - a, d)  # noqa: E731
+    parts = []
+    with fv.with_bf16_act(False):
+        for i in range(frames // fpb):
+            kw, vw = cache.update(0, r4(k, i * n, (i + 1) * n), r4(v, i * n, (i + 1) * n), i * n)
+            parts.append(fv.sdpa(r4(q, i * n, (i + 1) * n), kw, vw, fv.Plan.kv_window()))
+    torch.cuda.synchronize()
+    blocks = torch.cat(parts, dim=2).reshape(bh, s, d)
+    assert_parity(blocks.cpu().numpy(), whole.cpu().numpy(), "kv_blocks_vs_block_causal", max_abs=2e-3)
+    want = oracle.sdpa_composed(q, k, v, mask=oracle.block_causal_dense_mask(n, 0, 0, s, s))
+    assert_parity(blocks.cpu().numpy(), want, "kv_blocks_vs_oracle")
