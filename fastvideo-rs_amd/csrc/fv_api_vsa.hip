@@ -108,7 +108,9 @@ int fv_vdn_window_allows(size_t video_start, size_t frame_tokens, size_t frames,
     const size_t last = frames - 1;
     const size_t qf = (q - vs) / t, kf = (k - vs) / t;
     if (qf == 0 || kf == 0 || qf == last || kf == last) return 1;
-    const long long f = (long long)qf, c = (long long)chunk, r = (long long)radius, kk = (long long)kf;
+    // a radius or chunk past the clip reaches every frame: clamped so that the products stay in range
+    const long long f = (long long)qf, c = (long long)(chunk > frames ? frames : chunk),
+                    r = (long long)(radius > frames ? frames : radius), kk = (long long)kf;
     const long long lo = c > 0 ? (f / c - r) * c : f - r;
     const long long hi = c > 0 ? (f / c + r + 1) * c - 1 : f + r;
     return kk >= lo && kk <= hi;

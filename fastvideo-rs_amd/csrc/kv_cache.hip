@@ -22,6 +22,58 @@ __global__ __launch_bounds__(256) void kv_copy_rows_kernel(u32x4* __restrict__ d
     }
 }
 
+// Interleaved RoPE on BHSD rows (kernels/core.cu:1933-1955 `apply_rotary_bshd` through
+// wan/causal.rs:250-262 `rope_bhsd_f32`): pair (2i, 2i+1) of row r turns by the angle whose cos / sin
+// sit in the EVEN slot 2i of the [s, d] tables; f32 arithmetic, products unfused, as the reference.
+// One thread per 8 elements. Planes of x and out may be row windows of longer planes.
+template <bool IN16, bool OUT16>
+__global__ __launch_bounds__(256) void rope_bhsd_kernel(const void* __restrict__ x, size_t x_plane,
+                                                        const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                        float sin_sign, void* __restrict__ out, size_t out_plane,
+                                                        size_t s, size_t d, size_t total) {
+#pragma clang fp contract(off)
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const size_t du = d >> 3, u = i % du, row = (i / du) % s, bh = i / (du * s);
+    float v[8];
+    if constexpr (IN16) {
+        const u32x4 t = *reinterpret_cast<const u32x4*>((const uint16_t*)x + bh * x_plane + row * d + 8 * u);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[2 * j] = __builtin_bit_cast(float, t[j] << 16);
+            v[2 * j + 1] = __builtin_bit_cast(float, t[j] & 0xffff0000u);
+        }
+    } else {
+        const float* p = (const float*)x + bh * x_plane + row * d + 8 * u;
+        const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = a[j], v[4 + j] = b[j];
+    }
+    const float* cp = cos_t + row * d + 8 * u;
+    const float* sp = sin_t + row * d + 8 * u;
+    const f32x4 c0 = *reinterpret_cast<const f32x4*>(cp), c1 = *reinterpret_cast<const f32x4*>(cp + 4);
+    const f32x4 s0 = *reinterpret_cast<const f32x4*>(sp), s1 = *reinterpret_cast<const f32x4*>(sp + 4);
+    const float cs[4] = {c0[0], c0[2], c1[0], c1[2]};
+    const float sn[4] = {s0[0] * sin_sign, s0[2] * sin_sign, s1[0] * sin_sign, s1[2] * sin_sign};
+    float r[8];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float x1 = v[2 * j], x2 = v[2 * j + 1];
+        r[2 * j] = x1 * cs[j] - x2 * sn[j];
+        r[2 * j + 1] = x1 * sn[j] + x2 * cs[j];
+    }
+    if constexpr (OUT16) {
+        u32x4 t;
+#pragma unroll
+        for (int j = 0; j < 4; j++) t[j] = bf16_rne_bits(r[2 * j]) | ((unsigned)bf16_rne_bits(r[2 * j + 1]) << 16);
+        *reinterpret_cast<u32x4*>((uint16_t*)out + bh * out_plane + row * d + 8 * u) = t;
+    } else {
+        float* p = (float*)out + bh * out_plane + row * d + 8 * u;
+        *reinterpret_cast<f32x4*>(p) = f32x4{r[0], r[1], r[2], r[3]};
+        *reinterpret_cast<f32x4*>(p + 4) = f32x4{r[4], r[5], r[6], r[7]};
+    }
+}
+
 }  // namespace
 }  // namespace fv
 
@@ -92,32 +144,96 @@ int kv_shift_tokens_down(void* t, size_t rows, size_t from, size_t to, size_t le
     return FV_OK;
 }
 
+int kv_rope_bhsd(const void* x, DType x_dtype, size_t x_rows, const float* cos_t, const float* sin_t,
+                 bool negate_sin, void* out, DType out_dtype, size_t out_rows, size_t bh, size_t s, size_t d,
+                 hipStream_t st) {
+    if (!x || !cos_t || !sin_t || !out) return fv_invalid("rope_bhsd: null operand");
+    if (x_rows < s || out_rows < s) return fv_invalid("rope_bhsd: plane rows below the row count");
+    if (bh == 0 || s == 0) return FV_OK;
+    if (d == 0 || d % 8 != 0) return fv_decline("rope_bhsd: head dim must be a multiple of 8");
+    if ((((uintptr_t)x | (uintptr_t)out | (uintptr_t)cos_t | (uintptr_t)sin_t) & 15) != 0)
+        return fv_invalid("rope_bhsd: operands must be 16-byte aligned");
+    const size_t total = bh * s * (d / 8), blocks = (total + 255) / 256;
+    if (blocks > (size_t)INT_MAX) return fv_decline("rope_bhsd: too large for one launch");
+    const float sign = negate_sin ? -1.0f : 1.0f;
+    const dim3 grid((unsigned)blocks), block(256);
+    const bool i16 = x_dtype == DType::Bf16, o16 = out_dtype == DType::Bf16;
+#define FV_ROPE(I, O)                                                                                             \
+    hipLaunchKernelGGL((fv::rope_bhsd_kernel<I, O>), grid, block, 0, st, x, x_rows * d, cos_t, sin_t, sign, out, \
+                       out_rows * d, s, d, total)
+    if (i16 && o16) FV_ROPE(true, true);
+    else if (i16) FV_ROPE(true, false);
+    else if (o16) FV_ROPE(false, true);
+    else FV_ROPE(false, false);
+#undef FV_ROPE
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FV_OK : fv_fail_hip(e, "rope_bhsd");
+}
+
 CausalKvCache::CausalKvCache(KvSpec s, size_t num_layers) : spec(s), layers_(num_layers) {}
 
 CausalKvCache::~CausalKvCache() {
     for (auto& l : layers_) {
         if (l.k) (void)hipFree(l.k);
         if (l.v) (void)hipFree(l.v);
+        if (l.raw_sink) (void)hipFree(l.raw_sink);
     }
 }
 
 void CausalKvCache::reset() {
     std::lock_guard<std::mutex> g(mu_);
-    for (auto& l : layers_) l.global_end = l.local_end = 0;
+    for (auto& l : layers_) {
+        l.global_end = l.local_end = l.sink_at = 0;
+        l.raw_valid = false;
+    }
 }
 
 std::vector<KvPointers> CausalKvCache::pointers() const {
     std::lock_guard<std::mutex> g(mu_);
     std::vector<KvPointers> out;
-    for (const auto& l : layers_) out.push_back(KvPointers{l.global_end, l.local_end});
+    for (const auto& l : layers_) out.push_back(KvPointers{l.global_end, l.local_end, l.sink_at, l.raw_valid});
     return out;
+}
+
+Result<bool> CausalKvCache::set_pointers(const std::vector<KvPointers>& p) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (p.size() != layers_.size()) return kv_msg("causal kv: set_pointers needs a static cache and one entry per layer");
+    for (size_t i = 0; i < p.size(); i++) {
+        layers_[i].global_end = p[i].global_end;
+        layers_[i].local_end = p[i].local_end;
+        layers_[i].sink_at = p[i].sink_at;
+        layers_[i].raw_valid = p[i].raw_valid;
+    }
+    return true;
+}
+
+Result<bool> CausalKvCache::advance(size_t current_start, size_t n, size_t sink_target) {
+    std::lock_guard<std::mutex> g(mu_);
+    // plan every layer first, so that an error leaves no layer moved
+    std::vector<KvMove> moves;
+    for (const Layer& L : layers_) {
+        auto mv = kv_plan(spec, L.global_end, L.local_end, current_start, n);
+        if (!is_ok(mv)) return std::get<TensorError>(mv);
+        if (!L.k) return kv_msg("causal kv: advance over an unwritten cache");
+        moves.push_back(std::get<KvMove>(mv));
+    }
+    for (size_t i = 0; i < layers_.size(); i++) {
+        Layer& L = layers_[i];
+        if (spec.rebase_sink && spec.sink > 0 && sink_target > 0 && L.sink_at != sink_target && L.local_end >= spec.sink) {
+            L.raw_valid = true;
+            L.sink_at = sink_target;
+        }
+        L.global_end = current_start + n;
+        L.local_end = moves[i].local_end;
+    }
+    return true;
 }
 
 size_t CausalKvCache::bytes() const {
     std::lock_guard<std::mutex> g(mu_);
     size_t n = 0;
     for (const auto& l : layers_)
-        if (l.k) n += l.b * l.h * l.cap * (l.d * esize(l.kd) + l.dv * esize(l.vd));
+        if (l.k) n += l.b * l.h * (l.cap * (l.d * esize(l.kd) + l.dv * esize(l.vd)) + (l.raw_sink ? spec.sink * l.d * 4 : 0));
     return n;
 }
 
@@ -146,9 +262,12 @@ Result<std::pair<Tensor, Tensor>> CausalKvCache::update(size_t layer, const Tens
         if (b * h == 0 || cap == 0 || d == 0 || dv == 0) return kv_msg("causal kv: empty keys");
         hipError_t e = hipMalloc(&L.k, b * h * cap * d * esize(k.dtype));
         if (e == hipSuccess) e = hipMalloc(&L.v, b * h * cap * dv * esize(v.dtype));
+        if (e == hipSuccess && spec.rebase_sink && spec.sink > 0)
+            e = hipMalloc(&L.raw_sink, b * h * spec.sink * d * 4);   // f32, wan/causal.rs:650-655
         if (e != hipSuccess) {
             if (L.k) (void)hipFree(L.k);
-            L.k = L.v = nullptr;
+            if (L.v) (void)hipFree(L.v);
+            L.k = L.v = L.raw_sink = nullptr;
             return kv_msg(std::string("causal kv: allocating the layer's buffers: ") + hipGetErrorString(e));
         }
         L.b = b, L.h = h, L.cap = cap, L.d = d, L.dv = dv, L.kd = k.dtype, L.vd = v.dtype;
@@ -181,6 +300,32 @@ Result<std::pair<Tensor, Tensor>> CausalKvCache::update(size_t layer, const Tens
     Tensor kw = Tensor::window((char*)L.k + mv.window_start * d * esize(L.kd), {b, h, len, d}, L.kd, L.cap);
     Tensor vw = Tensor::window((char*)L.v + mv.window_start * dv * esize(L.vd), {b, h, len, dv}, L.vd, L.cap);
     return std::make_pair(std::move(kw), std::move(vw));
+}
+
+// wan/causal.rs:739-776 `rebase_sink`, static mode
+Result<bool> CausalKvCache::rebase_sink(size_t target, const float* orig_cos, const float* orig_sin,
+                                        const float* new_cos, const float* new_sin, hipStream_t st) {
+    std::lock_guard<std::mutex> g(mu_);
+    const size_t sink = spec.sink;
+    if (sink == 0) return false;
+    if (!spec.rebase_sink) return kv_msg("causal kv: rebase_sink needs the rebased-sink RoPE policy");
+    if (!orig_cos || !orig_sin || !new_cos || !new_sin) return kv_msg("causal kv: rebase_sink needs both table pairs");
+    bool any = false;
+    for (Layer& L : layers_) {
+        if (L.sink_at == target || !L.k || L.local_end < sink) continue;
+        if (!L.raw_sink) return kv_msg("causal kv: static rebased sink without its buffer");
+        const size_t bh = L.b * L.h;
+        int rc = FV_OK;
+        if (!L.raw_valid)   // rotating back by the sink's own positions recovers the un-roped keys, kept f32
+            rc = kv_rope_bhsd(L.k, L.kd, L.cap, orig_cos, orig_sin, true, L.raw_sink, DType::F32, sink, bh, sink, L.d, st);
+        if (rc == FV_OK)
+            rc = kv_rope_bhsd(L.raw_sink, DType::F32, sink, new_cos, new_sin, false, L.k, L.kd, L.cap, bh, sink, L.d, st);
+        if (rc != FV_OK) return kv_msg(std::string("causal kv: rebase_sink: ") + fv_sdpa_last_error());
+        L.raw_valid = true;
+        L.sink_at = target;
+        any = true;
+    }
+    return any;
 }
 
 }  // namespace fv::rt
@@ -222,11 +367,29 @@ int fv_kv_shift_tokens_down(void* t, size_t rows, size_t from, size_t to, size_t
 }
 
 fv_kv_cache* fv_kv_cache_new(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
-                             size_t layers) {
+                             int rope_policy, size_t layers) {
     fv::rt::KvSpec s;
     s.capacity = capacity, s.sink = sink, s.max_attention = max_attention, s.frame_tokens = frame_tokens;
     s.rolling = rolling != 0;
+    s.relativistic = rope_policy == FV_KV_ROPE_RELATIVISTIC;
+    s.rebase_sink = rope_policy == FV_KV_ROPE_REBASED_SINK && sink > 0;
     return new fv_kv_cache(s, layers);
+}
+
+int fv_rope_bhsd(const void* x, int x_is_bf16, size_t x_rows, const float* cos_t, const float* sin_t, int negate_sin,
+                 void* out, int out_is_bf16, size_t out_rows, size_t bh, size_t s, size_t d, void* stream) {
+    using fv::rt::DType;
+    return fv::rt::kv_rope_bhsd(x, x_is_bf16 ? DType::Bf16 : DType::F32, x_rows ? x_rows : s, cos_t, sin_t,
+                                negate_sin != 0, out, out_is_bf16 ? DType::Bf16 : DType::F32, out_rows ? out_rows : s,
+                                bh, s, d, (hipStream_t)stream);
+}
+
+int fv_kv_cache_rebase_sink(fv_kv_cache* c, size_t target, const float* orig_cos, const float* orig_sin,
+                            const float* new_cos, const float* new_sin, void* stream) {
+    if (!c) return fv_invalid("kv cache: null argument");
+    auto r = c->cache.rebase_sink(target, orig_cos, orig_sin, new_cos, new_sin, (hipStream_t)stream);
+    if (!fv::rt::is_ok(r)) return fv_invalid(std::get<fv::rt::TensorError>(r).message.c_str());
+    return FV_OK;
 }
 
 void fv_kv_cache_free(fv_kv_cache* c) { delete c; }
@@ -239,11 +402,29 @@ void fv_kv_cache_set_sink_guard(fv_kv_cache* c, int on) {
     if (c) c->cache.set_sink_guard(on != 0);
 }
 
-int fv_kv_cache_pointers(const fv_kv_cache* c, size_t layer, size_t out2[2]) {
-    if (!c || !out2) return fv_invalid("kv cache: null argument");
+int fv_kv_cache_pointers(const fv_kv_cache* c, size_t layer, size_t out4[4]) {
+    if (!c || !out4) return fv_invalid("kv cache: null argument");
     const auto p = c->cache.pointers();
     if (layer >= p.size()) return fv_invalid("causal kv: no such layer");
-    out2[0] = p[layer].global_end, out2[1] = p[layer].local_end;
+    out4[0] = p[layer].global_end, out4[1] = p[layer].local_end, out4[2] = p[layer].sink_at;
+    out4[3] = p[layer].raw_valid ? 1 : 0;
+    return FV_OK;
+}
+
+int fv_kv_cache_set_pointers(fv_kv_cache* c, const size_t* in4, size_t layers) {
+    if (!c || !in4) return fv_invalid("kv cache: null argument");
+    std::vector<fv::rt::KvPointers> p(layers);
+    for (size_t i = 0; i < layers; i++)
+        p[i] = fv::rt::KvPointers{in4[4 * i], in4[4 * i + 1], in4[4 * i + 2], in4[4 * i + 3] != 0};
+    auto r = c->cache.set_pointers(p);
+    if (!fv::rt::is_ok(r)) return fv_invalid(std::get<fv::rt::TensorError>(r).message.c_str());
+    return FV_OK;
+}
+
+int fv_kv_cache_advance(fv_kv_cache* c, size_t current_start, size_t n, size_t sink_target) {
+    if (!c) return fv_invalid("kv cache: null argument");
+    auto r = c->cache.advance(current_start, n, sink_target);
+    if (!fv::rt::is_ok(r)) return fv_invalid(std::get<fv::rt::TensorError>(r).message.c_str());
     return FV_OK;
 }
 

@@ -5,9 +5,10 @@
 // comes back as a row window of those buffers (no copy): the fused attention kernel reads a
 // (batch, head) plane at any plane stride.
 //
-// Built: absolute RoPE policy (keys arrive roped), rolling and global windows, the sink guard.
-// Not built: the relativistic and rebased-sink RoPE policies (they re-rope cached keys; the
-// constructor refuses them).
+// RoPE policies (wan/causal.rs:59-76): absolute (keys arrive roped); relativistic (the caller caches
+// un-roped keys and ropes the window itself at every forward: nothing for the cache to do but carry
+// the flag); rebased sink (absolute keys, the sink re-roped in place by `rebase_sink` from an f32
+// un-roped copy taken once).
 #pragma once
 #include <mutex>
 #include <utility>
@@ -23,6 +24,12 @@ struct KvSpec {
     size_t sink = 0;            // tokens kept at the head when the cache rolls
     size_t max_attention = 0;   // keys each query block reads, back from the end of the block
     bool rolling = false;       // a full cache drops its oldest tokens after the sink instead of refusing
+    bool relativistic = false;  // raw (normed, un-roped) keys cached; the window is roped by the caller
+    bool rebase_sink = false;   // absolute keys, the sink re-roped each block (`rebase_sink`)
+    // wan/causal.rs:136-145: the frame the sink keys should sit at once the write ending at frame
+    // end_frame is done, and the frames the queries can read
+    size_t window_frames() const { return max_attention / (frame_tokens ? frame_tokens : 1); }
+    size_t sink_target(size_t end_frame) const { return end_frame > window_frames() ? end_frame - window_frames() : 0; }
 };
 
 // wan/causal.rs:276-287
@@ -46,8 +53,17 @@ int kv_copy_tokens(void* dst, size_t dst_rows, size_t dst_off, const void* src, 
 int kv_shift_tokens_down(void* t, size_t rows, size_t from, size_t to, size_t len, size_t bh, size_t d,
                          DType dtype, hipStream_t st);
 
+// wan/causal.rs:250-262 `rope_bhsd_f32` / 264-274 `rope_bhsd`: interleaved RoPE (even-slot tables
+// [s, d]) of rows [0, s) of every plane of x into out; planes may be row windows (x_rows / out_rows
+// rows per plane); the result is f32 or rounded once to bf16.
+int kv_rope_bhsd(const void* x, DType x_dtype, size_t x_rows, const float* cos_t, const float* sin_t,
+                 bool negate_sin, void* out, DType out_dtype, size_t out_rows, size_t bh, size_t s, size_t d,
+                 hipStream_t st);
+
+// wan/causal.rs:353-360
 struct KvPointers {
-    size_t global_end = 0, local_end = 0;
+    size_t global_end = 0, local_end = 0, sink_at = 0;
+    bool raw_valid = false;
 };
 
 // wan/causal.rs:341-723, `new_static` mode.
@@ -63,10 +79,23 @@ class CausalKvCache {
     // [b, h, len, d] of the layer's buffers (plane_rows = capacity), valid until the next write.
     Result<std::pair<Tensor, Tensor>> update(size_t layer, const Tensor& k, const Tensor& v, size_t current_start,
                                              hipStream_t st);
+    // wan/causal.rs:733-806 `rebase_sink`: re-rope every layer's sink keys to start at frame `target`.
+    // orig_* are the tables of the sink's own frames [0, sink) (used once, to take the un-roped f32
+    // copy), new_* those of frames [target, target + sink): f32 [sink_tokens, d] each, even-slot.
+    // Returns whether any layer moved; a no-op where the sink is already there or not yet filled.
+    Result<bool> rebase_sink(size_t target, const float* orig_cos, const float* orig_sin, const float* new_cos,
+                             const float* new_sin, hipStream_t st);
     void reset();                         // a new rollout: pointers to zero, buffers (addresses) kept
     void set_sink_guard(bool on) { sink_guard_ = on; }
     bool sink_guard() const { return sink_guard_; }
     std::vector<KvPointers> pointers() const;
+    // wan/causal.rs:457-476 `set_pointers`: put pointers back (a graph replay moves no host state, a
+    // failed capture must leave none behind); one entry per layer.
+    Result<bool> set_pointers(const std::vector<KvPointers>& p);
+    // wan/causal.rs:503-536 `advance`: the host bookkeeping of one block forward of n tokens at
+    // current_start (sink target frame `sink_target`, 0: none) without its device work: what a graph
+    // replay of that forward leaves behind.
+    Result<bool> advance(size_t current_start, size_t n, size_t sink_target);
     size_t bytes() const;
     const KvSpec spec;
 
@@ -74,6 +103,9 @@ class CausalKvCache {
     struct Layer {
         void* k = nullptr;
         void* v = nullptr;
+        void* raw_sink = nullptr;   // f32 [b, h, sink, d], the un-roped sink keys
+        size_t sink_at = 0;
+        bool raw_valid = false;
         size_t b = 0, h = 0, cap = 0, d = 0, dv = 0;
         DType kd = DType::F32, vd = DType::F32;
         size_t global_end = 0, local_end = 0;

@@ -27,7 +27,11 @@ SIGNATURES = {
     "fv_kv_plan": (C.c_int, [_sz, _sz, _sz, _sz, C.c_int, _sz, _sz, _sz, _sz, _vp]),
     "fv_kv_copy_tokens": (C.c_int, [_vp, _sz, _sz, _vp, _sz, _sz, _sz, _sz, _sz, C.c_int, _vp]),
     "fv_kv_shift_tokens_down": (C.c_int, [_vp, _sz, _sz, _sz, _sz, _sz, _sz, C.c_int, _vp]),
-    "fv_kv_cache_new": (_vp, [_sz, _sz, _sz, _sz, C.c_int, _sz]),
+    "fv_kv_cache_new": (_vp, [_sz, _sz, _sz, _sz, C.c_int, C.c_int, _sz]),
+    "fv_kv_cache_rebase_sink": (C.c_int, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
+    "fv_kv_cache_set_pointers": (C.c_int, [_vp, _vp, _sz]),
+    "fv_kv_cache_advance": (C.c_int, [_vp, _sz, _sz, _sz]),
+    "fv_rope_bhsd": (C.c_int, [_vp, C.c_int, _sz, _vp, _vp, C.c_int, _vp, C.c_int, _sz, _sz, _sz, _sz, _vp]),
     "fv_kv_cache_free": (None, [_vp]),
     "fv_kv_cache_reset": (None, [_vp]),
     "fv_kv_cache_set_sink_guard": (None, [_vp, C.c_int]),

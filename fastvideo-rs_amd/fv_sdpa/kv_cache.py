@@ -10,7 +10,7 @@ import torch
 from . import _lib
 from .sdpa import TensorError, _desc, _FvTensor
 
-__all__ = ["KvSpec", "KvMove", "CausalKvCache", "kv_copy_tokens", "kv_shift_tokens_down"]
+__all__ = ["KvSpec", "KvMove", "KvRope", "CausalKvCache", "kv_copy_tokens", "kv_shift_tokens_down", "rope_bhsd"]
 
 
 class KvMove:
@@ -23,20 +23,35 @@ class KvMove:
         return f"KvMove(evicted={self.evicted}, local=[{self.local_start}, {self.local_end}), window_start={self.window_start})"
 
 
-class KvSpec:
-    """wan/causal.rs:38-57 (absolute RoPE policy only)."""
+class KvRope:
+    """wan/causal.rs:59-76."""
+    ABSOLUTE, RELATIVISTIC, REBASED_SINK = 0, 1, 2
 
-    def __init__(self, frame_tokens, capacity, sink, max_attention, rolling):
+
+class KvSpec:
+    """wan/causal.rs:38-57."""
+
+    def __init__(self, frame_tokens, capacity, sink, max_attention, rolling, rope=KvRope.ABSOLUTE):
         self.frame_tokens, self.capacity, self.sink = int(frame_tokens), int(capacity), int(sink)
         self.max_attention, self.rolling = int(max_attention), bool(rolling)
+        self.relativistic = rope == KvRope.RELATIVISTIC
+        self.rebase_sink = rope == KvRope.REBASED_SINK and self.sink > 0
+
+    @property
+    def rope(self):
+        return KvRope.RELATIVISTIC if self.relativistic else (KvRope.REBASED_SINK if self.rebase_sink else KvRope.ABSOLUTE)
 
     @staticmethod
-    def rolling_window(frame_tokens, local_attn_frames, sink_frames):
-        """wan/causal.rs:110-131 `KvSpec::rolling` with KvRope::Absolute."""
+    def rolling_window(frame_tokens, local_attn_frames, sink_frames, rope=KvRope.ABSOLUTE):
+        """wan/causal.rs:110-131 `KvSpec::rolling`."""
         if local_attn_frames == 0 or sink_frames >= local_attn_frames:
             raise TensorError(f"causal kv: sink {sink_frames} frames must be below the window ({local_attn_frames} frames)")
         n = local_attn_frames * frame_tokens
-        return KvSpec(frame_tokens, n, sink_frames * frame_tokens, n, True)
+        return KvSpec(frame_tokens, n, sink_frames * frame_tokens, n, True, rope)
+
+    def sink_target(self, end_frame):
+        """wan/causal.rs:136-138."""
+        return max(end_frame - self.window_frames(), 0)
 
     @staticmethod
     def global_window(frame_tokens, frames, sink_frames=0):
@@ -75,8 +90,9 @@ class CausalKvCache:
 
     def __init__(self, spec, num_layers):
         self.spec = spec
+        self._layers = num_layers
         self._h = _lib.lib().fv_kv_cache_new(spec.capacity, spec.sink, spec.max_attention, spec.frame_tokens,
-                                             int(spec.rolling), num_layers)
+                                             int(spec.rolling), spec.rope, num_layers)
         if not self._h:
             raise TensorError("causal kv: could not create the cache")
 
@@ -114,9 +130,40 @@ class CausalKvCache:
         _lib.lib().fv_kv_cache_set_sink_guard(self._h, int(bool(on)))
 
     def pointers(self, layer=0):
-        out = (C.c_size_t * 2)()
+        """(global_end, local_end) of a layer."""
+        return self.pointers4(layer)[:2]
+
+    def pointers4(self, layer=0):
+        """(global_end, local_end, sink_at, raw_valid) of a layer (wan/causal.rs:353-360)."""
+        out = (C.c_size_t * 4)()
         _lib.check(_lib.lib().fv_kv_cache_pointers(self._h, layer, out))
-        return int(out[0]), int(out[1])
+        return int(out[0]), int(out[1]), int(out[2]), bool(out[3])
+
+    def set_pointers(self, per_layer):
+        """wan/causal.rs:457-476: one (global_end, local_end, sink_at, raw_valid) per layer."""
+        flat = (C.c_size_t * (4 * len(per_layer)))(*[int(x) for p in per_layer for x in p])
+        lib = _lib.lib()
+        if lib.fv_kv_cache_set_pointers(self._h, flat, len(per_layer)) != 0:
+            raise TensorError(lib.fv_sdpa_last_error().decode())
+
+    def advance(self, current_start, n, sink_target=0):
+        """wan/causal.rs:503-536: the bookkeeping of one block forward without its device work."""
+        lib = _lib.lib()
+        if lib.fv_kv_cache_advance(self._h, current_start, n, sink_target) != 0:
+            raise TensorError(lib.fv_sdpa_last_error().decode())
+
+    def rebase_sink(self, target, orig, new):
+        """wan/causal.rs:733-776: re-rope every layer's sink keys to start at frame `target`;
+        orig / new = (cos, sin) f32 [sink_tokens, d] tables of the sink's own frames / of the target's."""
+        for t in (*orig, *new):
+            if not (t.is_cuda and t.is_contiguous() and t.dtype == torch.float32 and t.dim() == 2
+                    and t.shape[0] == self.spec.sink):
+                raise ValueError("rebase_sink: tables must be contiguous f32 [sink_tokens, d] CUDA tensors")
+        lib = _lib.lib()
+        rc = lib.fv_kv_cache_rebase_sink(self._h, target, orig[0].data_ptr(), orig[1].data_ptr(), new[0].data_ptr(),
+                                         new[1].data_ptr(), torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise TensorError(lib.fv_sdpa_last_error().decode())
 
     def bytes(self):
         return int(_lib.lib().fv_kv_cache_bytes(self._h))
@@ -145,3 +192,20 @@ def kv_shift_tokens_down(t, frm, to, length):
     _lib.check(_lib.lib().fv_kv_shift_tokens_down(t.data_ptr(), t.shape[1], frm, to, length, t.shape[0], t.shape[2],
                                                   int(t.dtype == torch.bfloat16),
                                                   torch.cuda.current_stream().cuda_stream))
+
+
+def rope_bhsd(x, cos, sin, negate_sin=False, out_bf16=None):
+    """wan/causal.rs:250-274 `rope_bhsd_f32` (out_bf16=False) / `rope_bhsd` (x's dtype): interleaved RoPE
+    of x [b, h, s, d] (f32 or bf16, contiguous) with even-slot tables [s, d]."""
+    if not (x.is_cuda and x.is_contiguous() and x.dim() == 4 and x.dtype in (torch.float32, torch.bfloat16)):
+        raise ValueError("rope_bhsd: want a contiguous [b, h, s, d] CUDA tensor of f32 or bf16")
+    b, h, s, d = x.shape
+    for t in (cos, sin):
+        if not (t.is_cuda and t.is_contiguous() and t.dtype == torch.float32 and tuple(t.shape) == (s, d)):
+            raise ValueError(f"rope_bhsd: tables must be contiguous f32 [{s}, {d}]")
+    o16 = (x.dtype == torch.bfloat16) if out_bf16 is None else bool(out_bf16)
+    out = torch.empty((b, h, s, d), device=x.device, dtype=torch.bfloat16 if o16 else torch.float32)
+    _lib.check(_lib.lib().fv_rope_bhsd(x.data_ptr(), int(x.dtype == torch.bfloat16), s, cos.data_ptr(), sin.data_ptr(),
+                                       int(bool(negate_sin)), out.data_ptr(), int(o16), s, b * h, s, d,
+                                       torch.cuda.current_stream().cuda_stream))
+    return out

@@ -162,23 +162,44 @@ int fv_kv_copy_tokens(void* dst, size_t dst_rows, size_t dst_off, const void* sr
 int fv_kv_shift_tokens_down(void* t, size_t rows, size_t from, size_t to, size_t len, size_t bh, size_t d,
                             int is_bf16, void* stream);
 /* wan/causal.rs:341-723 `CausalKvCache::new_static`: one persistent [b, h, capacity, d] K / V pair per
- * layer (allocated with hipMalloc at the layer's first write, kept by fv_kv_cache_reset). The RoPE
- * policy is the absolute one (keys arrive roped); the relativistic and rebased-sink policies are not
- * built. fv_kv_cache_update = `update`: rolls (wan/causal.rs:678-690), writes the block's k / v
+ * layer (allocated with hipMalloc at the layer's first write, kept by fv_kv_cache_reset). rope_policy
+ * (wan/causal.rs:59-76 `KvRope`): absolute (keys arrive roped), relativistic (the caller caches
+ * un-roped keys and ropes the window itself; the cache only carries the flag), rebased sink (absolute
+ * keys, the sink re-roped in place by fv_kv_cache_rebase_sink). fv_kv_cache_update = `update`: rolls (wan/causal.rs:678-690), writes the block's k / v
  * [b, h, n, d] at current_start and returns the windows the block's queries read as row windows of
  * the layer's buffers (plane_rows = capacity; valid until the layer's next update): pass them to
  * fv_rt_sdpa with FV_PLAN_KV_WINDOW (or fv_sdpa_dense_bf16_strided). Errors carry the reference's
  * messages. One cache is driven from one thread at a time per layer (a mutex serialises the host
  * bookkeeping); the device work is ordered on `stream`. */
 typedef struct fv_kv_cache fv_kv_cache;
+enum { FV_KV_ROPE_ABSOLUTE = 0, FV_KV_ROPE_RELATIVISTIC = 1, FV_KV_ROPE_REBASED_SINK = 2 };
 fv_kv_cache* fv_kv_cache_new(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
-                             size_t layers);
+                             int rope_policy, size_t layers);
 void fv_kv_cache_free(fv_kv_cache* c);
 void fv_kv_cache_reset(fv_kv_cache* c);
 /* wan/causal.rs:396-418 `set_sink_guard`: a write that re-runs cached frames leaves the sink slots. */
 void fv_kv_cache_set_sink_guard(fv_kv_cache* c, int on);
-/* out2 = {global_end, local_end} of a layer (wan/causal.rs:431-445 `pointers`). */
-int fv_kv_cache_pointers(const fv_kv_cache* c, size_t layer, size_t out2[2]);
+/* out4 = {global_end, local_end, sink_at, raw_valid} of a layer (wan/causal.rs:353-360, 431-445). */
+int fv_kv_cache_pointers(const fv_kv_cache* c, size_t layer, size_t out4[4]);
+/* wan/causal.rs:457-476 `set_pointers`: in4 = `layers` x {global_end, local_end, sink_at, raw_valid}, one
+ * entry per layer of the cache (a HIP-graph replay of a block forward moves no host state). */
+int fv_kv_cache_set_pointers(fv_kv_cache* c, const size_t* in4, size_t layers);
+/* wan/causal.rs:503-536 `advance`: the host bookkeeping of one block forward of n tokens at current_start
+ * (rebased-sink target frame sink_target, 0: none) on every layer, without its device work. */
+int fv_kv_cache_advance(fv_kv_cache* c, size_t current_start, size_t n, size_t sink_target);
+/* wan/causal.rs:733-776 `rebase_sink` (static mode): re-rope every layer's sink keys to start at frame
+ * `target`. orig_cos / orig_sin: tables of the sink's own frames (used once, to take the un-roped f32
+ * copy by rotating back); new_cos / new_sin: tables of frames [target, target + sink): f32
+ * [sink_tokens, d], even-slot, device memory. Layers already there, or not yet holding the sink, are
+ * left alone. */
+int fv_kv_cache_rebase_sink(fv_kv_cache* c, size_t target, const float* orig_cos, const float* orig_sin,
+                            const float* new_cos, const float* new_sin, void* stream);
+/* wan/causal.rs:250-274 `rope_bhsd_f32` / `rope_bhsd` (kernels/core.cu:1933-1955 `apply_rotary_bshd` on
+ * BHSD): out[:, r, 2i] = x1*c - x2*s, out[:, r, 2i+1] = x1*s + x2*c for rows r < s of every plane, c / s
+ * from the even slot 2i of the f32 [s, d] tables (negate_sin: the inverse rotation). x / out are f32 or
+ * bf16 bits (the bf16 result is the f32 one rounded once), planes x_rows / out_rows rows apart (0 = s). */
+int fv_rope_bhsd(const void* x, int x_is_bf16, size_t x_rows, const float* cos_t, const float* sin_t, int negate_sin,
+                 void* out, int out_is_bf16, size_t out_rows, size_t bh, size_t s, size_t d, void* stream);
 size_t fv_kv_cache_bytes(const fv_kv_cache* c);
 int fv_kv_cache_update(fv_kv_cache* c, size_t layer, const fv_tensor* k, const fv_tensor* v, size_t current_start,
                        fv_tensor* k_window, fv_tensor* v_window, void* stream);

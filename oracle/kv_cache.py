@@ -10,17 +10,39 @@ through the cache == the whole clip under the block-causal mask).
 """
 import numpy as np
 
-__all__ = ["KvSpecO", "KvError", "CausalKvCacheO"]
+__all__ = ["KvSpecO", "KvError", "CausalKvCacheO", "rope_bhsd_f32"]
 
 
 class KvError(ValueError):
     pass
 
 
+def rope_bhsd_f32(x, cos, sin):
+    """causal.rs:250-262 over `apply_rotary_bshd` (C/rt/ops.rs:1903-1935): pair (2i, 2i+1) of row r of
+    every [b, h] plane turns by the angle whose cos / sin sit in the EVEN slot 2i of the [s, d] tables.
+    f32 arithmetic, each product rounded before the sum."""
+    x = np.asarray(x, dtype=np.float32)
+    c = np.asarray(cos, dtype=np.float32)[None, None, :, 0::2]
+    s = np.asarray(sin, dtype=np.float32)[None, None, :, 0::2]
+    x1, x2 = x[..., 0::2], x[..., 1::2]
+    out = np.empty_like(x)
+    out[..., 0::2] = (x1 * c).astype(np.float32) - (x2 * s).astype(np.float32)
+    out[..., 1::2] = (x1 * s).astype(np.float32) + (x2 * c).astype(np.float32)
+    return out
+
+
 class KvSpecO:
-    def __init__(self, frame_tokens, capacity, sink, max_attention, rolling):
+    def __init__(self, frame_tokens, capacity, sink, max_attention, rolling, rebase_sink=False):
         self.frame_tokens, self.capacity, self.sink = frame_tokens, capacity, sink
         self.max_attention, self.rolling = max_attention, rolling
+        self.rebase_sink = rebase_sink and sink > 0
+
+    def window_frames(self):
+        return self.max_attention // max(self.frame_tokens, 1)
+
+    def sink_target(self, end_frame):
+        """causal.rs:136-138."""
+        return max(end_frame - self.window_frames(), 0)
 
     def plan(self, global_end, local_end_prev, current_start, n):
         """causal.rs:289-336 -> (evicted, local_start, local_end, window_start)."""
@@ -48,8 +70,8 @@ class KvSpecO:
 
 class _Layer:
     def __init__(self):
-        self.k = self.v = None
-        self.global_end = self.local_end = 0
+        self.k = self.v = self.raw_sink = None
+        self.global_end = self.local_end = self.sink_at = 0
 
 
 class CausalKvCacheO:
@@ -60,6 +82,24 @@ class CausalKvCacheO:
 
     def reset(self):
         self.layers = [_Layer() for _ in self.layers]
+
+    def rebase_sink(self, target, orig, new, quantize=None):
+        """causal.rs:733-808 (tensor-per-write path): re-rope every layer's sink keys to start at frame
+        `target`; orig / new = (cos, sin) [sink_tokens, d] of the sink's own frames / the target's.
+        quantize: the rounding of a bf16 cache (None for f32)."""
+        sink = self.spec.sink
+        if sink == 0:
+            return
+        for slot in self.layers:
+            if slot.sink_at == target or slot.k is None or slot.k.shape[2] < sink:
+                continue
+            if slot.raw_sink is None:
+                slot.raw_sink = rope_bhsd_f32(slot.k[:, :, :sink], orig[0], -np.asarray(orig[1], dtype=np.float32))
+            head = rope_bhsd_f32(slot.raw_sink, new[0], new[1])
+            if quantize is not None:
+                head = quantize(head)
+            slot.k = np.concatenate([head, slot.k[:, :, sink:]], axis=2)
+            slot.sink_at = target
 
     def update(self, layer, k, v, current_start):
         slot, spec = self.layers[layer], self.spec

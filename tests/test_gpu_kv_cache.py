@@ -127,6 +127,29 @@ def test_cache_windows_equal_the_oracles(fv, oracle, case, bf16):
     assert np.array_equal(kw.float().cpu().numpy(), ocache.update(0, rnd(k), rnd(v), 0)[0])
 
 
+def test_update_keeps_prefix_and_window(fv):
+    """The reference's known answers for `update` (causal.rs:1111-1152), each token's value repeated
+    over a 4-wide head dim (the device copies move 16-byte units)."""
+    import torch
+
+    announce("kv cache known answers")
+    cache = fv.CausalKvCache(fv.KvSpec(2, 8, 2, 8, True), 1)
+    blk = lambda base: (base + torch.arange(4, dtype=torch.float32, device="cuda")).reshape(1, 1, 4, 1).repeat(1, 1, 1, 4)  # noqa: E731
+
+    def flat(w):
+        torch.cuda.synchronize()
+        assert torch.equal(w, w[..., :1].expand_as(w))
+        return w[0, 0, :, 0].tolist()
+
+    assert flat(cache.update(0, blk(0.0), blk(0.0), 0)[0]) == [0.0, 1.0, 2.0, 3.0]
+    assert flat(cache.update(0, blk(10.0), blk(10.0), 0)[0]) == [10.0, 11.0, 12.0, 13.0]
+    assert cache.update(0, blk(20.0), blk(20.0), 4)[0].shape[2] == 8
+    assert flat(cache.update(0, blk(30.0), blk(30.0), 8)[0]) == [10.0, 11.0, 22.0, 23.0, 30.0, 31.0, 32.0, 33.0]
+    assert cache.pointers(0)[1] == 8
+    kw, vw = cache.update(0, blk(40.0), blk(40.0), 12)        # 1-token... the roll moves 2 tokens by 4
+    assert flat(kw) == [10.0, 11.0, 32.0, 33.0, 40.0, 41.0, 42.0, 43.0] and flat(vw) == flat(kw)
+
+
 def test_cache_errors_and_sink_guard(fv, oracle):
     import torch
 
@@ -221,3 +244,87 @@ def test_cached_blocks_equal_the_masked_whole_clip(fv, oracle):
     assert_parity(blocks.cpu().numpy(), whole.cpu().numpy(), "kv_blocks_vs_block_causal", max_abs=2e-3)
     want = oracle.sdpa_composed(q, k, v, mask=oracle.block_causal_dense_mask(n, 0, 0, s, s))
     assert_parity(blocks.cpu().numpy(), want, "kv_blocks_vs_oracle")
+
+
+def _rope_tables(seed, s, d, frame0=0.0):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    theta = rng.uniform(0.01, 1.0, (1, d // 2)) * (np.arange(s)[:, None] + frame0)
+    return (np.repeat(np.cos(theta), 2, axis=1).astype(np.float32), np.repeat(np.sin(theta), 2, axis=1).astype(np.float32))
+
+
+@pytest.mark.parametrize("in16", [False, True])
+@pytest.mark.parametrize("out16", [False, True])
+def test_rope_bhsd_bit_exact(fv, oracle, in16, out16):
+    import torch
+
+    announce(f"rope_bhsd in16={in16} out16={out16}")
+    b, h, s, d = 2, 3, 37, 64
+    rng = np.random.Generator(np.random.PCG64(21))
+    x = rng.standard_normal((b, h, s, d)).astype(np.float32)
+    if in16:
+        x = oracle.quantize_bf16(x)
+    cos, sin = _rope_tables(22, s, d)
+    tx = torch.from_numpy(x).cuda().to(torch.bfloat16 if in16 else torch.float32)
+    tc, ts = torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda()
+    for neg in (False, True):
+        want = oracle.rope_bhsd_f32(x, cos, -sin if neg else sin)
+        if out16:
+            want = oracle.quantize_bf16(want)
+        got = fv.rope_bhsd(tx, tc, ts, negate_sin=neg, out_bf16=out16)
+        torch.cuda.synchronize()
+        assert got.dtype == (torch.bfloat16 if out16 else torch.float32)
+        assert np.array_equal(got.float().cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_rebased_sink_policy_equals_the_oracles(fv, oracle, bf16):
+    """A rolling cache under the rebased-sink RoPE policy (causal.rs:733-776): after every roll the
+    sink is re-roped to the frames just before the rolled part; cache contents equal the oracle's bit
+    for bit (the rope is elementwise f32), pointers follow, advance / set_pointers move host state only."""
+    import torch
+
+    announce(f"kv rebased sink bf16={bf16}")
+    b, h, d, ft, layers = 1, 2, 64, 4, 2
+    win_f, sink_f, blk_f = 6, 2, 2
+    n, sink = blk_f * ft, sink_f * ft
+    spec = fv.KvSpec.rolling_window(ft, win_f, sink_f, fv.KvRope.REBASED_SINK)
+    ospec = oracle.KvSpecO(ft, win_f * ft, sink, win_f * ft, True, rebase_sink=True)
+    cache, ocache = fv.CausalKvCache(spec, layers), oracle.CausalKvCacheO(ospec, layers)
+    dt = torch.bfloat16 if bf16 else torch.float32
+    rnd = oracle.quantize_bf16 if bf16 else (lambda x: x)
+    dev = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+    cos_o, sin_o = _rope_tables(30, sink, d)
+    for blk in range(6):
+        end_frame = (blk + 1) * blk_f
+        target = spec.sink_target(end_frame)
+        assert target == ospec.sink_target(end_frame)
+        if target > 0:
+            cos_n, sin_n = _rope_tables(30, sink, d, frame0=float(target * ft))
+            cache.rebase_sink(target, (dev(cos_o), dev(sin_o)), (dev(cos_n), dev(sin_n)))
+            ocache.rebase_sink(target, (cos_o, sin_o), (cos_n, sin_n), quantize=rnd if bf16 else None)
+        for layer in range(layers):
+            k, v = _blocks(40 + 10 * layer + blk, b, h, n, d, 1)[0]
+            k, v = rnd(k), rnd(v)
+            want_k, want_v = ocache.update(layer, k, v, blk * n)
+            kw, vw = cache.update(layer, dev(k).to(dt), dev(v).to(dt), blk * n)
+            torch.cuda.synchronize()
+            assert np.array_equal(kw.float().cpu().numpy(), want_k), (blk, layer)
+            assert np.array_equal(vw.float().cpu().numpy(), want_v), (blk, layer)
+            o = ocache.layers[layer]
+            # a layer's sink moves at the first rebase after it holds the sink
+            assert cache.pointers4(layer)[:3] == (o.global_end, o.local_end, o.sink_at)
+    assert cache.pointers4(0)[3] is True
+    # advance == update's bookkeeping without device work; set_pointers puts a state back
+    state = [cache.pointers4(layer) for layer in range(layers)]
+    cache.advance(6 * n, n, spec.sink_target(7 * blk_f))
+    moved = cache.pointers4(0)
+    assert moved[0] == 7 * n and moved[2] == spec.sink_target(7 * blk_f)
+    cache.set_pointers(state)
+    assert [cache.pointers4(layer) for layer in range(layers)] == state
+    with pytest.raises(fv.TensorError, match="one entry per layer"):
+        cache.set_pointers(state[:1])
+    plain = fv.CausalKvCache(fv.KvSpec.rolling_window(ft, win_f, sink_f), 1)
+    with pytest.raises(fv.TensorError, match="rebased-sink RoPE policy"):
+        plain.rebase_sink(1, (dev(cos_o), dev(sin_o)), (dev(cos_o), dev(sin_o)))
+    with pytest.raises(fv.TensorError, match="advance over an unwritten cache"):
+        plain.advance(0, n)

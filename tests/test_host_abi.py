@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), name
     assert fv_sdpa.lib().fv_sdpa_arch() == b"gfx950"
-    assert fv_sdpa.lib().fv_sdpa_last_error() == b""
+    assert isinstance(fv_sdpa.lib().fv_sdpa_last_error(), bytes)   # "" until a call of this thread fails
 
 
 def test_supported_table():

@@ -103,3 +103,69 @@ def test_oracle_cache_rolls_by_hand(oracle):
     c2.sink_guard = True
     kw, _ = c2.update(0, 50 + tok(0, 4), tok(0, 4), 0)        # current_start == 0: not a recompute, lands whole
     assert seen(kw)[:4] == [50, 51, 52, 53]
+
+
+def test_update_keeps_prefix_and_window(oracle):
+    """The reference's known answers, causal.rs:1111-1152 (2-token frames, capacity 8, sink 2)."""
+    c = oracle.CausalKvCacheO(oracle.KvSpecO(2, 8, 2, 8, True), 1)
+    blk = lambda base: (base + np.arange(4, dtype=np.float32)).reshape(1, 1, 4, 1)  # noqa: E731
+    flat = lambda w: w.reshape(-1).tolist()  # noqa: E731
+    assert flat(c.update(0, blk(0.0), blk(0.0), 0)[0]) == [0.0, 1.0, 2.0, 3.0]
+    assert flat(c.update(0, blk(10.0), blk(10.0), 0)[0]) == [10.0, 11.0, 12.0, 13.0]      # next step: overwritten
+    assert c.update(0, blk(20.0), blk(20.0), 4)[0].shape[2] == 8
+    assert flat(c.update(0, blk(30.0), blk(30.0), 8)[0]) == [10.0, 11.0, 22.0, 23.0, 30.0, 31.0, 32.0, 33.0]
+    assert c.layers[0].local_end == 8
+    assert flat(c.update(0, blk(40.0), blk(40.0), 12)[0]) == [10.0, 11.0, 32.0, 33.0, 40.0, 41.0, 42.0, 43.0]
+
+
+def _tables(seed, s, d, frame0=0.0):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    theta = (rng.uniform(0.01, 1.0, (1, d // 2)) * (np.arange(s)[:, None] + frame0)).astype(np.float64)
+    return (np.repeat(np.cos(theta), 2, axis=1).astype(np.float32), np.repeat(np.sin(theta), 2, axis=1).astype(np.float32), theta)
+
+
+def test_rope_bhsd_is_a_rotation_of_pairs(oracle):
+    """causal.rs:250-262: against the complex-number closed form in f64, norm of every pair kept, the
+    inverse rotation (sin negated) undoes it, angle 0 is the identity, tables read from the EVEN slot."""
+    rng = np.random.Generator(np.random.PCG64(9))
+    b, h, s, d = 2, 3, 7, 16
+    x = rng.standard_normal((b, h, s, d)).astype(np.float32)
+    cos, sin, theta = _tables(1, s, d)
+    got = oracle.rope_bhsd_f32(x, cos, sin)
+    z = (x[..., 0::2].astype(np.float64) + 1j * x[..., 1::2].astype(np.float64)) * np.exp(1j * theta)[None, None]
+    assert np.abs(got[..., 0::2] - z.real).max() < 1e-6 and np.abs(got[..., 1::2] - z.imag).max() < 1e-6
+    n_in = x[..., 0::2] ** 2 + x[..., 1::2] ** 2
+    n_out = got[..., 0::2] ** 2 + got[..., 1::2] ** 2
+    assert np.allclose(n_in, n_out, rtol=1e-5)
+    back = oracle.rope_bhsd_f32(got, cos, -sin)
+    assert np.abs(back - x).max() < 1e-6
+    assert np.array_equal(oracle.rope_bhsd_f32(x, np.ones_like(cos), np.zeros_like(sin)), x)
+    # the odd slots of the tables are never read
+    cos2, sin2 = cos.copy(), sin.copy()
+    cos2[:, 1::2], sin2[:, 1::2] = 123.0, -7.0
+    assert np.array_equal(oracle.rope_bhsd_f32(x, cos2, sin2), got)
+
+
+def test_rebased_sink_lands_where_roping_there_directly_would(oracle):
+    """causal.rs:733-808: the sink keys, roped at frames [0, sink), are re-roped to frames
+    [target, target + sink) through an un-roped f32 copy taken once: equal (to rounding) to roping the
+    raw keys at the target frames directly, and moving twice does not compound error."""
+    rng = np.random.Generator(np.random.PCG64(10))
+    b, h, d, ft = 1, 2, 16, 3
+    spec = oracle.KvSpecO(ft, 6 * ft, 2 * ft, 6 * ft, True, rebase_sink=True)
+    raw = rng.standard_normal((b, h, 6 * ft, d)).astype(np.float32)
+    cos0, sin0, _ = _tables(2, 6 * ft, d)                       # positions 0 .. 6*ft of the clip
+    c = oracle.CausalKvCacheO(spec, 1)
+    c.update(0, oracle.rope_bhsd_f32(raw, cos0, sin0), raw, 0)
+    sink = spec.sink
+    assert spec.sink_target(9) == 3 and spec.sink_target(5) == 0
+    for target in (3, 7, 3):
+        cosn, sinn, _ = _tables(2, sink, d, frame0=float(target * ft))
+        c.rebase_sink(target, (cos0[:sink], sin0[:sink]), (cosn, sinn))
+        want = oracle.rope_bhsd_f32(raw[:, :, :sink], cosn, sinn)
+        assert np.abs(c.layers[0].k[:, :, :sink] - want).max() < 2e-6
+        assert np.array_equal(c.layers[0].k[:, :, sink:], oracle.rope_bhsd_f32(raw, cos0, sin0)[:, :, sink:])
+        assert c.layers[0].sink_at == target
+    before = c.layers[0].k.copy()
+    c.rebase_sink(3, (cos0[:sink], sin0[:sink]), (cosn, sinn))   # already there: untouched
+    assert np.array_equal(c.layers[0].k, before)
