@@ -366,16 +366,30 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
 extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 
 namespace {
+// The kernel's dynamic LDS limit (128 KB at D = 128), once per device.
 template <bool MASKED, int D>
-hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
+hipError_t flash_attr() {
     static std::atomic<unsigned long long> attr_done;
     constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
-    hipError_t e = fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<MASKED, D>, lds, attr_done);
+    return fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<MASKED, D>, lds, attr_done);
+}
+template <bool MASKED, int D>
+hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
+    constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
+    hipError_t e = flash_attr<MASKED, D>();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((fv::flash_fwd_pp2<MASKED, D>), dim3(p->per_xcd * 8), dim3(512), lds, stream, *p);
     return hipGetLastError();
 }
 }  // namespace
+
+extern "C" hipError_t fv_internal_init_flash(void) {
+    hipError_t e = flash_attr<false, 128>();
+    if (e == hipSuccess) e = flash_attr<true, 128>();
+    if (e == hipSuccess) e = flash_attr<false, 64>();
+    if (e == hipSuccess) e = flash_attr<true, 64>();
+    return e;
+}
 
 extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int masked, int d,
                                                hipStream_t stream) {

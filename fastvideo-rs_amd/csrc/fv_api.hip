@@ -137,6 +137,12 @@ extern "C" {
 const char* fv_sdpa_last_error(void) { return g_last_error.c_str(); }
 const char* fv_sdpa_arch(void) { return "gfx950"; }
 
+int fv_sdpa_init(void) {
+    hipError_t e = fv_internal_init_flash();
+    if (e == hipSuccess) e = fv_internal_init_vsa();
+    return e == hipSuccess ? FV_OK : fail_hip(e, "fv_sdpa_init");
+}
+
 int fv_sdpa_supported(size_t b, size_t h, size_t sq, size_t sk, size_t d) {
     if (b != 0 && h > (size_t)65535 / b) return 0;
     const size_t bh = b * h;

@@ -66,6 +66,8 @@ extern "C" hipError_t fv_internal_launch_topk(const float* scores, unsigned* out
 extern "C" hipError_t fv_internal_launch_tile_qkv(const void* x, int x_is_bf16, const int* slot_src,
                                                   uint16_t* xt, size_t bh, size_t seq, size_t padded,
                                                   int dim, hipStream_t st);
+extern "C" hipError_t fv_internal_init_flash(void);
+extern "C" hipError_t fv_internal_init_vsa(void);
 extern "C" hipError_t fv_internal_launch_fine(const fv::VsaFineParams* p, hipStream_t st);
 extern "C" hipError_t fv_internal_launch_combine(const float* sparse, const float* coarse,
                                                  const void* gate, int gate_is_bf16,

@@ -535,6 +535,13 @@ extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16,
     return hipGetLastError();
 }
 
+// The coarse PV kernel's dynamic LDS limit (8 rows of up to 4096 scores), once per device.
+extern "C" hipError_t fv_internal_init_vsa(void) {
+    static std::atomic<unsigned long long> attr_done;
+    return fv_set_max_lds_once((const void*)vsa_coarse_pv_kernel, (int)(sizeof(float) * kCoarseRows * kTopkMaxN),
+                               attr_done);
+}
+
 extern "C" hipError_t fv_internal_launch_coarse(const float* qc, const float* kc, const float* vc,
                                                 float* scores, float* coarse, size_t bh, int nb,
                                                 int dim, float scale, hipStream_t st) {
@@ -543,9 +550,7 @@ extern "C" hipError_t fv_internal_launch_coarse(const float* qc, const float* kc
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || !coarse) return e;
     const size_t lds = sizeof(float) * kCoarseRows * (size_t)nb;
-    static std::atomic<unsigned long long> attr_done;
-    e = fv_set_max_lds_once((const void*)vsa_coarse_pv_kernel, (int)(sizeof(float) * kCoarseRows * kTopkMaxN),
-                            attr_done);
+    e = fv_internal_init_vsa();
     if (e != hipSuccess) return e;
     const dim3 g2((nb + kCoarseRows - 1) / kCoarseRows, (unsigned)bh);
     hipLaunchKernelGGL(vsa_coarse_pv_kernel, g2, dim3(256), lds, st, scores, vc, coarse, nb);

@@ -43,6 +43,7 @@ SIGNATURES = {
     "fv_cast_f32_bf16": (C.c_int, [_vp, _vp, _sz, _vp]),
     "fv_cast_bf16_f32": (C.c_int, [_vp, _vp, _sz, _vp]),
     "fv_sdpa_composed_f32": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _vp, _sz, _sz, _sz, _sz, C.c_float, _vp]),
+    "fv_sdpa_init": (C.c_int, []),
     "fv_rt_sdpa": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "fv_rt_free": (C.c_int, [_vp, _vp]),
     "fv_rt_set_bf16_activations": (None, [C.c_int]),

@@ -32,6 +32,13 @@ const char* fv_sdpa_last_error(void);
 /* "gfx950" — the only code object in the library. */
 const char* fv_sdpa_arch(void);
 
+/* Per-device set-up of the current HIP device: raises the dynamic-LDS limit of the kernels that use
+ * more than 64 KB (`hipFuncSetAttribute`, the reference's `opt_in_dynamic_shared`, rt/ops.rs:1445-1461).
+ * Optional: every entry point does this itself at its first launch on a device; call it before
+ * capturing a HIP graph whose first launch of a kernel would otherwise fall inside the capture.
+ * Idempotent, thread-safe. */
+int fv_sdpa_init(void);
+
 /* rt/attn.rs:112-128 `mma_sdpa_supported`: 1 when the fused kernel takes a
  * [b,h,sq,d] x [b,h,sk,d] call: d == 128 or d == 64, sq > 0, sk > 0,
  * 1 <= b*h <= 65535, lengths fit int32. */

@@ -1,8 +1,8 @@
 """HIP-graph capture of the library's entry points: every call is stream-ordered and allocates
 nothing, so a captured call replays on new data in the same buffers. Each graph is replayed several
 times with eager work and synchronisations of the program's own in between, and every replay is
-checked bit for bit against the eager call on the same inputs. (The once-per-device LDS attribute of
-a kernel is set at its first eager launch, so each kernel runs eagerly once before its capture.)
+checked bit for bit against the eager call on the same inputs. (`fv_sdpa_init` sets the once-per-device
+LDS attributes of the kernels up front, so that no capture has to.)
 """
 import numpy as np
 import pytest
@@ -19,7 +19,8 @@ def fv():
     assert torch.cuda.is_available()
     import fv_sdpa
 
-    fv_sdpa.lib()
+    assert fv_sdpa.lib().fv_sdpa_init() == 0   # per-device kernel attributes, before any capture
+    assert fv_sdpa.lib().fv_sdpa_init() == 0   # idempotent
     return fv_sdpa
 
 
