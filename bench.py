@@ -8,7 +8,7 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache) are for the
+Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache|composed) are for the
 design notes; the driver's line is the default `self`.
 """
 import argparse
@@ -200,6 +200,56 @@ def bench_kvcache(args):
     print(json.dumps(rec), flush=True)
 
 
+def bench_composed(args):
+    """The composed f32 SDPA on the device (masked plans, Plan::composed, fallbacks): H=12, S=4096,
+    d=128, f32 operands and a shared additive block-causal mask [S, S]; all arithmetic fp32 on the
+    matrix cores (v_mfma_f32_32x32x2_f32: 157.3 TFLOP/s peak)."""
+    import torch
+
+    import fv_sdpa
+
+    lib = fv_sdpa.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    h, s, d = 12, 4096, 128
+    g = torch.Generator(device=dev).manual_seed(20244)
+    q, k, v = (torch.randn((h, s, d), generator=g, device=dev) for _ in range(3))
+    blk = torch.arange(s, device=dev) // 512
+    mask = torch.where(blk[None, :] <= blk[:, None], 0.0, -1e9).to(torch.float32).contiguous()
+    out = torch.empty_like(q)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        rc = lib.fv_sdpa_composed_f32(q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), 0, out.data_ptr(), h, s,
+                                      s, d, 1.0 / d ** 0.5, stream)
+        if rc != 0:
+            raise RuntimeError(lib.fv_sdpa_last_error().decode())
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in evs:
+        a.record()
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / args.steps
+    avg = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    flops = 4.0 * h * s * s * d     # every pair is computed (the mask is additive)
+    tf = flops / (avg * 1e-3) / 1e12
+    rec = {
+        "metric": "composed f32 SDPA TFLOP/s (H=12 S=4096 d=128, additive mask)", "value": round(flops / (wall * 1e-3) / 1e12, 3),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "composed f32 SDPA with a shared additive [S, S] mask, H=12 S=4096 d=128", "flops_per_call": flops},
+        "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
+                     "traffic": None, "kernel": "fv::sdpa_composed_mfma_f32_kernel<128>", "avg_kernel_ms": round(avg, 4)},
+    }
+    print(json.dumps(rec), flush=True)
+
+
 def bench_prep(args):
     """The producer / consumer either side of the SDPA call at the headline shape: q and k
     RMSNorm + RoPE (bf16 kernel) and the V split out of a fused bf16 QKV projection
@@ -334,7 +384,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache"])
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "composed"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -361,6 +411,9 @@ def main():
         return
     if args.workload == "kvcache":
         bench_kvcache(args)
+        return
+    if args.workload == "composed":
+        bench_composed(args)
         return
     fv_sdpa.lib()
     dev = torch.device("cuda:0")

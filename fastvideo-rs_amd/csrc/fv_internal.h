@@ -66,6 +66,10 @@ extern "C" hipError_t fv_internal_launch_topk(const float* scores, unsigned* out
 extern "C" hipError_t fv_internal_launch_tile_qkv(const void* x, int x_is_bf16, const int* slot_src,
                                                   uint16_t* xt, size_t bh, size_t seq, size_t padded,
                                                   int dim, hipStream_t st);
+// 1 = launched, 0 = not this kernel's head dim / alignment, < 0 = -(hipError_t)
+extern "C" int fv_internal_launch_composed_mfma(const float* q, const float* k, const float* v, const float* mask,
+                                                long mask_bh_stride, float* out, size_t bh, int sq, int sk, int d,
+                                                float scale, hipStream_t st);
 extern "C" hipError_t fv_internal_init_flash(void);
 extern "C" hipError_t fv_internal_init_vsa(void);
 extern "C" hipError_t fv_internal_launch_fine(const fv::VsaFineParams* p, hipStream_t st);

@@ -17,8 +17,8 @@
 
 // ---- composed SDPA on the device (rt/sdpa.rs:328-342) ----------------------------------
 // softmax(scale * q k^T + mask) v in f32, one workgroup per query row, online
-// softmax over chunks of 256 keys. The fallback for masked calls and for shapes
-// the fused kernel declines; not a fast path.
+// softmax over chunks of 256 keys: the scalar form, for the head dims the f32 matrix-core kernel
+// (composed_fwd.hip: 32 / 64 / 96 / 128) does not take.
 namespace fv {
 
 constexpr int kCompThreads = 256;
@@ -96,6 +96,11 @@ extern "C" int fv_sdpa_composed_f32(const float* q, const float* k, const float*
     if (sk == 0) return fv_invalid("sdpa_composed: no keys");
     if (d == 0 || d > 256 || bh > 65535 || sq > (size_t)INT_MAX || sk > (size_t)INT_MAX)
         return fv_decline("sdpa_composed: needs 1 <= d <= 256, bh <= 65535, lengths < 2^31");
+    // head dims 32 / 64 / 96 / 128: the f32 matrix-core kernel (composed_fwd.hip)
+    const int rc = fv_internal_launch_composed_mfma(q, k, v, mask, mask_per_bh ? (long)(sq * sk) : 0L, out, bh, (int)sq,
+                                                    (int)sk, (int)d, scale, (hipStream_t)stream);
+    if (rc < 0) return fv_fail_hip((hipError_t)(-rc), "sdpa_composed_mfma_f32");
+    if (rc == 1) return FV_OK;
     hipLaunchKernelGGL(fv::sdpa_composed_f32_kernel, dim3((unsigned)sq, (unsigned)bh), dim3(fv::kCompThreads), 0,
                        (hipStream_t)stream, q, k, v, mask, mask_per_bh ? (long)(sq * sk) : 0L, out, (int)sq,
                        (int)sk, (int)d, scale);

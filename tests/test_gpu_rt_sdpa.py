@@ -189,7 +189,12 @@ def test_block_causal_and_kv_window_plans_at_d128(fv, oracle):
 
 
 @pytest.mark.parametrize("bh,sq,sk,d,mask_kind", [(2, 5, 7, 8, None), (3, 33, 300, 64, "shared"), (2, 40, 257, 128, "per_bh"),
-                                                  (1, 3, 1000, 256, None), (2, 64, 64, 128, "shared"), (1, 2, 1, 128, None)])
+                                                  (1, 3, 1000, 256, None), (2, 64, 64, 128, "shared"), (1, 2, 1, 128, None),
+                                                  # the f32 matrix-core kernel: every head dim it takes, query / key tails,
+                                                  # one and many key tiles, more than one workgroup per head
+                                                  (2, 300, 515, 32, "shared"), (3, 129, 31, 96, None), (2, 257, 1025, 96, "per_bh"),
+                                                  (1, 128, 32, 128, None), (2, 700, 333, 128, "shared"), (4, 1, 65, 64, "per_bh"),
+                                                  (1, 384, 2048, 128, None)])
 def test_composed_kernel_vs_oracle(fv, oracle, bh, sq, sk, d, mask_kind):
     import ctypes
     import torch
