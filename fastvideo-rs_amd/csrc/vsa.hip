@@ -382,22 +382,26 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
     SoftmaxState st;
     st.init();
 
-    int tile = min((int)sel[0], nb - 1);
-    tile_load_async<2, false>(kbuf, kb + (size_t)tile * kTileElems * 128, kTileElems, wave, lane);
+    // Per-lane DMA offsets are loop-invariant (every tile has 64 rows in the tile-ordered layout), so a
+    // tile load is 8 (m0, load) pairs from a scalar base. The tile indices and sizes of the next two
+    // list entries are fetched one iteration ahead: no scalar-load latency sits in front of a DMA issue.
+    TileDma<2, 128> dma;
+    dma.init(wave, lane);
+    auto tile_at = [&](int i) -> int { return min((int)sel[min(i, topk - 1)], nb - 1); };
+    int tile = tile_at(0), tile_next = tile_at(1);
+    int valid = p.block_sizes[tile], valid_next = p.block_sizes[tile_next];
+    dma.template issue<false>(kbuf, kb + (size_t)tile * kTileElems * 128, kTileElems, wave);
 #pragma unroll 1
     for (int i = 0; i < topk; i++) {
-        const int valid = p.block_sizes[tile];
         wait_vmcnt<0>();     // K(i) landed
         block_barrier();     // ... for every wave; PV(i-1) finished everywhere: V buffer free
-        tile_load_async<2, true>(vbuf, vb + (size_t)tile * kTileElems * 128, kTileElems, wave, lane);
+        dma.template issue<true>(vbuf, vb + (size_t)tile * kTileElems * 128, kTileElems, wave);
+        const int tile_nn = tile_at(i + 2);          // consumed an iteration from now
         f32x16 s[2];
         qk_tile(kbuf, rb.k, qf, s);
         block_barrier();     // K buffer free
         const bool more = i + 1 < topk;
-        if (more) {
-            tile = min((int)sel[i + 1], nb - 1);
-            tile_load_async<2, false>(kbuf, kb + (size_t)tile * kTileElems * 128, kTileElems, wave, lane);
-        }
+        if (more) dma.template issue<false>(kbuf, kb + (size_t)tile_next * kTileElems * 128, kTileElems, wave);
         if (valid < kTileElems) {
 #pragma unroll
             for (int b = 0; b < 2; b++)
@@ -412,6 +416,10 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
         if (more) wait_vmcnt<8>(); else wait_vmcnt<0>();   // V(i) landed; K(i+1) may be in flight
         block_barrier();
         pv_tile(vbuf, rb.v, pb, o);
+        tile = tile_next;
+        tile_next = tile_nn;
+        valid = valid_next;
+        valid_next = p.block_sizes[tile_nn];
     }
 
     const float l_tot = pair_sum(st.l_acc);
