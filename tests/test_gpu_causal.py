@@ -117,3 +117,25 @@ def test_headline_causal_shape_sampled_rows(fv, oracle, bt):
     want = oracle.sdpa_composed_rows(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), rows,
                                      mask_bc=(bt, 0, 0))
     assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, f"causal_headline_{bt}")
+
+
+@pytest.mark.parametrize("mode", ["block_causal", "vdn_window"])
+def test_full_size_masked_rows_of_ones(fv, mode):
+    """With V = 1 every row of a masked call is 1 if its visible weights are normalised right: a check
+    of the whole full-size output (tile walks, boundary masks, longest-first order) without an oracle."""
+    import torch
+
+    bh, d = 12, 128
+    s = 32760 if mode == "block_causal" else 49920
+    announce(f"masked rows-of-ones {mode} bh={bh} s={s}")
+    g = torch.Generator(device="cuda").manual_seed(12)
+    q, k = (torch.randn((bh, s, d), generator=g, device="cuda", dtype=torch.bfloat16) for _ in range(2))
+    v = torch.ones((bh, s, d), device="cuda", dtype=torch.bfloat16)
+    if mode == "block_causal":
+        out = fv.sdpa_block_causal_bf16(q, k, v, 1560, 0, 0)
+    else:
+        out = fv.sdpa_vdn_window_bf16(q, k, v, 0, 1560, 32, 5, 1)
+    torch.cuda.synchronize()
+    err = (out - 1.0).abs().max().item()
+    print(f"max |out - 1| = {err:.3e}")
+    assert err <= 4e-3

@@ -164,3 +164,46 @@ def test_headline_shape_sampled_rows(fv, oracle):
     torch.cuda.synchronize()
     wantc = oracle.sdpa_composed_rows(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), rows)
     assert_parity(outc[:, torch.from_numpy(rows).cuda()].cpu().numpy(), wantc, "cross_headline_rows")
+
+
+def test_wan14b_shape_sampled_rows(fv, oracle):
+    """Wan-14B 720p self- and cross-attention at full size (H = 40, S = 75600, Sk = 512): parity on
+    sampled rows; the whole sequence of every head is resident on the one GPU."""
+    import torch
+
+    bh, s, d = 40, 75600, 128
+    announce(f"dense wan14b bh={bh} s={s}")
+    g = torch.Generator(device="cuda").manual_seed(2025)
+    q, k, v = (torch.randn((bh, s, d), generator=g, device="cuda", dtype=torch.bfloat16) for _ in range(3))
+    out = fv.sdpa_dense_bf16(q, k, v, out_bf16=True)
+    torch.cuda.synchronize()
+    rows = sample_rows(5, s, 12, extra=(0, 255, 256, s - 1))
+    ridx = torch.from_numpy(rows).cuda()
+    heads = [0, 7, 19, 39]      # the oracle walks 75600 keys per row: four heads keep it in seconds
+    hk = lambda x: x[heads].float().cpu().numpy()  # noqa: E731
+    want = oracle.sdpa_composed_rows(hk(q), hk(k), hk(v), rows)
+    assert_parity(out[heads][:, ridx].float().cpu().numpy(), want, "wan14b_self_rows", max_abs=2e-2)
+    kc, vc = k[:, :512].contiguous(), v[:, :512].contiguous()
+    outc = fv.sdpa_dense_bf16(q, kc, vc)
+    torch.cuda.synchronize()
+    wantc = oracle.sdpa_composed_rows(hk(q), hk(kc), hk(vc), rows)
+    assert_parity(outc[heads][:, ridx].cpu().numpy(), wantc, "wan14b_cross_rows")
+
+
+@pytest.mark.parametrize("bh,s", [(12, 32760), (40, 75600)])
+def test_full_size_rows_of_ones(fv, bh, s):
+    """A property every row of the full-size call must keep, checked on the whole output: with V = 1 the
+    softmax weights of a row sum to one, so the output is 1 wherever the weights are normalised right
+    (tile tails, rescales, the last partial query tile)."""
+    import torch
+
+    d = 128
+    announce(f"dense rows-of-ones bh={bh} s={s}")
+    g = torch.Generator(device="cuda").manual_seed(11)
+    q, k = (torch.randn((bh, s, d), generator=g, device="cuda", dtype=torch.bfloat16) for _ in range(2))
+    v = torch.ones((bh, s, d), device="cuda", dtype=torch.bfloat16)
+    out = fv.sdpa_dense_bf16(q, k, v)
+    torch.cuda.synchronize()
+    err = (out - 1.0).abs().max().item()
+    print(f"max |out - 1| = {err:.3e}")
+    assert err <= 4e-3     # P is rounded to bf16 (2^-9 relative) before it meets V; l sums the unrounded P

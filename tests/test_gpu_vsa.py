@@ -326,3 +326,25 @@ def test_headline_vsa_shapes(fv, oracle, grid, topk):
             want_rows.append(coarse[None, :] * gn[b, toks[qt]] + sparse)
             got_rows.append(outn[b, toks[qt]])
     assert_parity(np.concatenate(got_rows), np.concatenate(want_rows), f"vsa_headline_{grid}")
+
+
+@pytest.mark.parametrize("grid,sparsity", [((21, 30, 52), 0.8), ((32, 32, 32), 0.875)])
+def test_full_size_rows_of_ones(fv, grid, sparsity):
+    """V = 1 and a zero gate at the two full-size geometries: the fine stage's softmax over the selected
+    tiles' real tokens sums to one, so every real token's output is 1 (partial tiles, padding slots and
+    the scatter back to token order included); with gate = 1 the coarse branch adds its own 1."""
+    import torch
+
+    announce(f"vsa rows-of-ones grid={grid}")
+    ctx = fv.VsaCtx(grid, sparsity)
+    heads = 12
+    g = torch.Generator(device="cuda").manual_seed(13)
+    q, k = (torch.randn((heads, ctx.seq, D), generator=g, device="cuda").to(torch.bfloat16) for _ in range(2))
+    v = torch.ones((heads, ctx.seq, D), device="cuda", dtype=torch.bfloat16)
+    scale = float(1.0 / np.sqrt(D))
+    out0 = fv.vsa_attention_device(q, k, v, torch.zeros_like(v), ctx, scale)
+    out1 = fv.vsa_attention_device(q, k, v, None, ctx, scale)
+    torch.cuda.synchronize()
+    e0, e1 = (out0 - 1.0).abs().max().item(), (out1 - 2.0).abs().max().item()
+    print(f"max |out - 1| = {e0:.3e} (zero gate), max |out - 2| = {e1:.3e} (gate of one)")
+    assert e0 <= 4e-3 and e1 <= 4e-3
