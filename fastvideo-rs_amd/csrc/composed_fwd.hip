@@ -199,6 +199,7 @@ extern "C" int fv_internal_launch_composed_mfma(const float* q, const float* k, 
                                                 long mask_bh_stride, float* out, size_t bh, int sq, int sk, int d,
                                                 float scale, hipStream_t st) {
     if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0) return 0;
+    if (sk > INT_MAX - 2 * fv::kCK || sq > INT_MAX - fv::kCQ) return 0;   // tile indices stay in int range
     hipError_t e;
     switch (d) {
         case 32: e = fv::launch_composed<32>(q, k, v, mask, mask_bh_stride, out, bh, sq, sk, scale, st); break;
