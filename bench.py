@@ -8,7 +8,7 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache|composed) are for the
+Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache|kvcache1|composed) are for the
 design notes; the driver's line is the default `self`.
 """
 import argparse
@@ -130,12 +130,14 @@ def bench_vsa(args):
     print(json.dumps(rec), flush=True)
 
 
-def bench_kvcache(args):
-    """Autoregressive Self-Forcing self-attention of one layer: 7 blocks of 3 latent frames (4680
-    tokens) written into a 21-frame KV cache and each block's queries attending the cache window in
-    place (Plan::kv_window). One step = the whole 7-block rollout of the layer: 7 cache writes + 7
-    dense calls of Sq = 4680 against Sk = 4680 ... 32760. The same with a contiguous copy of every
-    window first (what the reference's `narrow` does) is timed beside it."""
+def bench_kvcache(args, fpb=3):
+    """Autoregressive Self-Forcing self-attention of one layer: blocks of `fpb` latent frames (3: 4680
+    tokens, the reference's geometry; 1: 1560 tokens) written into a 21-frame KV cache and each block's
+    queries attending the cache window in place (Plan::kv_window). One step = the whole rollout of the
+    layer: 21/fpb cache writes + dense calls of Sq = fpb*1560 against Sk = Sq ... 32760, with the keys
+    split over several workgroups where the query tiles alone do not fill the GPU (the library's own
+    choice, fv_sdpa_splitkv_choose). The same with a contiguous copy of every window first (what the
+    reference's `narrow` does) and without split-KV is timed beside it."""
     import torch
 
     import fv_sdpa
@@ -143,7 +145,7 @@ def bench_kvcache(args):
     lib = fv_sdpa.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    h, d, ft, fpb, frames = 12, 128, 1560, 3, 21
+    h, d, ft, frames = 12, 128, 1560, 21
     n, blocks = fpb * ft, frames // fpb
     g = torch.Generator(device=dev).manual_seed(20243)
     qs, ks, vs = ([torch.randn((1, h, n, d), generator=g, device=dev).to(torch.bfloat16) for _ in range(blocks)]
@@ -154,7 +156,11 @@ def bench_kvcache(args):
     outs = [torch.empty((h, n, d), device=dev, dtype=torch.bfloat16) for _ in range(blocks)]
     scale = 1.0 / d ** 0.5
 
-    def rollout(copy_windows):
+    ws_bytes = max(int(lib.fv_sdpa_splitkv_workspace_bytes(h, n, d, 16)), 256)
+    ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+    splits_used = []
+
+    def rollout(copy_windows, split=True):
         cache.reset()
         for i in range(blocks):
             kw, vw = cache.update(0, ks[i], vs[i], i * n)
@@ -162,8 +168,11 @@ def bench_kvcache(args):
                 kw, vw = kw.contiguous(), vw.contiguous()
             sk = kw.shape[2]
             rows = kw.stride(1) // d
-            rc = lib.fv_sdpa_dense_bf16_strided(qs[i].data_ptr(), kw.data_ptr(), vw.data_ptr(), outs[i].data_ptr(), 1,
-                                                h, n, sk, d, scale, 0, rows, rows, stream)
+            sp = int(lib.fv_sdpa_splitkv_choose(h, n, sk)) if split else 1
+            if len(splits_used) < blocks and split and not copy_windows:
+                splits_used.append(sp)
+            rc = lib.fv_sdpa_dense_bf16_splitkv(qs[i].data_ptr(), kw.data_ptr(), vw.data_ptr(), outs[i].data_ptr(), 1,
+                                                h, n, sk, d, scale, 0, rows, rows, sp, ws.data_ptr(), ws_bytes, stream)
             if rc != 0:
                 raise RuntimeError(lib.fv_sdpa_last_error().decode())
 
@@ -178,7 +187,8 @@ def bench_kvcache(args):
         return (time.perf_counter() - t0) * 1e3 / args.steps
 
     in_place = timed(lambda: rollout(False))
-    copied = timed(lambda: rollout(True))
+    copied = timed(lambda: rollout(True, split=False))
+    unsplit = timed(lambda: rollout(False, split=False))
     # the plan entry once, to show it takes the same route
     kw, vw = cache.update(0, ks[0], vs[0], 0)
     before = fv_sdpa.rt_stats()
@@ -191,9 +201,10 @@ def bench_kvcache(args):
         "value": round(tf, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(in_place, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "7 blocks x 4680 queries against a 21-frame KV cache (Sk = 4680 ... 32760), H=12 d=128, "
-                               "cache write + attention per block", "flops_per_step": flops},
-        "ms_per_step_with_window_copies": round(copied, 4),
+        "config": {"workload": f"{blocks} blocks x {n} queries against a 21-frame KV cache (Sk = {n} ... 32760), H=12 d=128, "
+                               "cache write + attention per block", "flops_per_step": flops,
+                   "key_splits_per_block": splits_used},
+        "ms_per_step_with_window_copies_no_split": round(copied, 4), "ms_per_step_in_place_no_split": round(unsplit, 4),
         "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::flash_fwd_pp2<false, 128>"},
     }
@@ -384,7 +395,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "composed"])
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "kvcache1", "composed"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -409,8 +420,8 @@ def main():
     if args.workload == "prep":
         bench_prep(args)
         return
-    if args.workload == "kvcache":
-        bench_kvcache(args)
+    if args.workload in ("kvcache", "kvcache1"):
+        bench_kvcache(args, 3 if args.workload == "kvcache" else 1)
         return
     if args.workload == "composed":
         bench_composed(args)

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     // sequence): longest first over the whole launch, tile index major and head minor
     // (block-causal: last tile first; VDN window: the anchor / global tiles at both ends
     // first); measured 9 % faster than the dense order, whose per-XCD ranges hold unequal work.
-    int bh, qt;
+    int bh, qt, sp = 0;   // sp: this workgroup's key split (dense launches with kv_split > 1)
     if constexpr (MASKED) {
         const int work = blockIdx.x;
         if (work >= p.total) return;
@@ -94,8 +94,11 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     } else {
         const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
         if (work >= p.total) return;
-        bh = work / p.nqt;
-        qt = work % p.nqt;
+        const int per_bh = p.nqt * p.kv_split;
+        bh = work / per_bh;
+        const int rem = work - bh * per_bh;
+        qt = rem / p.kv_split;
+        sp = rem - qt * p.kv_split;
     }
     const int q0 = qt * kPpBM;
     const int sq = p.sq, sk = p.sk;
@@ -114,7 +117,10 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     const uint16_t* Kh = p.k + (size_t)bh * p.k_plane;
     const uint16_t* Vh = p.v + (size_t)bh * p.v_plane;
 
-    const int nkt = (sk + kBN - 1) / kBN;
+    const int nkt_all = (sk + kBN - 1) / kBN;
+    // a split walks key tiles [t0, t0 + nkt) of the nkt_all tiles (the whole range without split-KV)
+    const int t0 = MASKED ? 0 : sp * p.split_tiles;
+    const int nkt = MASKED ? nkt_all : min(p.split_tiles, nkt_all - t0);
     // The key-tile walk of this query tile: up to three ascending tile ranges [a_i, a_i + n_i),
     // n0 + n1 + n2 = ne tiles in all. A lane's query sees key x iff
     //   x < a_hi  ||  x >= c_lo  ||  (w_lo <= x && x < w_hi).
@@ -182,7 +188,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     auto kv0_of = [&](int e) -> int {
         e = min(e, ne - 1);
         if constexpr (MASKED) return (e < n0 ? e : e < n0 + n1 ? a1 + (e - n0) : a2 + (e - n0 - n1)) * kBN;
-        else return e * kBN;
+        else return (t0 + e) * kBN;
     };
     // tile t lives in buffer t mod 4 (t >= -2)
     auto kbuf = [&](int t) -> lds_u8* { return smem + (t & (kRing2 - 1)) * kTileBytes; };
@@ -339,6 +345,26 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     const float l_tot = pair_sum(st.l_acc);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int row = wave * 32 + c32;
+    if constexpr (!MASKED) {
+        if (p.kv_split > 1) {
+            // partial result of this split: O / l in f32 and log2 of the sum of 2^(s * sl2) it covers
+            if (row < qlen) {
+                const size_t prow = ((size_t)sp * (p.total / (p.nqt * p.kv_split)) + bh) * sq + q0 + row;
+                float* po = p.part_o + prow * kD;
+#pragma unroll
+                for (int db = 0; db < kNO; db++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        f32x4 r;
+#pragma unroll
+                        for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
+                        *reinterpret_cast<f32x4*>(po + 32 * db + 8 * g + 4 * h) = r;
+                    }
+                if (h == 0) p.part_lse[prow] = l_tot > 0.f ? st.ms_used + __builtin_log2f(l_tot) : NEG;
+            }
+            return;
+        }
+    }
     if (row < qlen) {
         const size_t base = ((size_t)bh * sq + q0 + row) * kD;
 #pragma unroll
@@ -359,7 +385,55 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     }
 }
 
+// Merge of the split-KV partials: out[row] = sum_s w_s O_s / sum_s w_s with w_s = 2^(lse_s - max lse).
+// One thread per (row, 4 d).
+template <bool OUT16>
+__global__ __launch_bounds__(256) void splitkv_merge_kernel(const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_lse, void* __restrict__ out,
+                                                            size_t rows, int d, int splits) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const int d4 = d >> 2;
+    if (i >= rows * d4) return;
+    const size_t row = i / d4;
+    const int c = (int)(i - row * d4) * 4;
+    float m = neg_inf();
+    for (int s = 0; s < splits; s++) m = __builtin_fmaxf(m, part_lse[(size_t)s * rows + row]);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float wsum = 0.f;
+    if (m != neg_inf()) {
+        for (int s = 0; s < splits; s++) {
+            const float w = fast_exp2(part_lse[(size_t)s * rows + row] - m);
+            const f32x4 o = *reinterpret_cast<const f32x4*>(part_o + ((size_t)s * rows + row) * d + c);
+            wsum += w;
+#pragma unroll
+            for (int x = 0; x < 4; x++) acc[x] += w * o[x];
+        }
+    }
+    const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+#pragma unroll
+    for (int x = 0; x < 4; x++) acc[x] *= inv;
+    if constexpr (OUT16) {
+        *reinterpret_cast<bf16x4*>((uint16_t*)out + row * d + c) = __builtin_convertvector(acc, bf16x4);
+    } else {
+        *reinterpret_cast<f32x4*>((float*)out + row * d + c) = acc;
+    }
+}
+
 }  // namespace fv
+
+extern "C" hipError_t fv_internal_launch_splitkv_merge(const float* part_o, const float* part_lse, void* out,
+                                                       int out_is_bf16, size_t rows, int d, int splits,
+                                                       hipStream_t st) {
+    const size_t n = rows * (size_t)(d / 4), blocks = (n + 255) / 256;
+    if (blocks == 0) return hipSuccess;
+    if (out_is_bf16)
+        hipLaunchKernelGGL(fv::splitkv_merge_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, part_o, part_lse,
+                           out, rows, d, splits);
+    else
+        hipLaunchKernelGGL(fv::splitkv_merge_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, part_o, part_lse,
+                           out, rows, d, splits);
+    return hipGetLastError();
+}
 
 // ---- host launchers -------------------------------------------------------------
 

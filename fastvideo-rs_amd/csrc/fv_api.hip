@@ -56,6 +56,9 @@ enum { kMaskNone = 0, kMaskBlockCausal = 1, kMaskVdnWindow = 2 };
 struct MaskArgs {
     int mode = kMaskNone;
     size_t q_rows = 0, k_rows = 0, v_rows = 0;   // rows per (batch, head) plane; 0 = contiguous (sq / sk)
+    size_t splits = 1;                            // split-KV (dense only): key splits per query tile
+    void* workspace = nullptr;                    // ... and their partial results
+    size_t workspace_bytes = 0;
     size_t block_tokens = 0, window = 0, sink = 0;                           // block-causal
     size_t video_start = 0, frame_tokens = 0, frames = 0, chunk = 0, radius = 0;   // VDN window
 };
@@ -125,8 +128,35 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
         if (m.frames <= 2) mode = kMaskNone;   // anchors only: dense
     }
     p.mask_mode = mode;
+    p.kv_split = 1;
+    p.split_tiles = INT_MAX;
+    p.part_o = nullptr;
+    p.part_lse = nullptr;
+    const size_t nkt = (sk + 63) / 64;
+    size_t splits = mode == kMaskNone ? m.splits : 1;
+    if (splits > 1) {
+        const size_t per = (nkt + splits - 1) / splits;
+        splits = (nkt + per - 1) / per;             // no empty split
+        if (splits > 1) {
+            if (total * splits > (size_t)INT_MAX / 2) return decline("sdpa: too many workgroups for one launch");
+            const size_t need = fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits);
+            if (!m.workspace || m.workspace_bytes < need || (((uintptr_t)m.workspace) & 255) != 0)
+                return fv_invalid("sdpa: split-KV needs a 256-byte aligned workspace of fv_sdpa_splitkv_workspace_bytes");
+            p.kv_split = (int)splits;
+            p.split_tiles = (int)per;
+            p.part_o = (float*)m.workspace;
+            p.part_lse = (float*)((char*)m.workspace + ((splits * bh * sq * d * 4 + 255) & ~(size_t)255));
+            p.total = (int)(total * splits);
+            p.per_xcd = (p.total + 7) / 8;
+        }
+    }
     hipError_t e = fv_internal_launch_flash(&p, mode != kMaskNone ? 1 : 0, (int)d, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip(e, mode != kMaskNone ? "flash_fwd_pp2<masked>" : "flash_fwd_pp2<dense>");
+    if (p.kv_split > 1) {
+        e = fv_internal_launch_splitkv_merge(p.part_o, p.part_lse, out, out_is_bf16 ? 1 : 0, bh * sq, (int)d, p.kv_split,
+                                             (hipStream_t)stream);
+        if (e != hipSuccess) return fail_hip(e, "splitkv_merge");
+    }
     return FV_OK;
 }
 
@@ -163,6 +193,54 @@ int fv_sdpa_dense_bf16_strided(const uint16_t* q, const uint16_t* k, const uint1
     m.q_rows = q_rows;
     m.k_rows = k_rows;
     m.v_rows = v_rows;
+    return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, m, stream);
+}
+
+size_t fv_sdpa_splitkv_workspace_bytes(size_t bh, size_t sq, size_t d, size_t splits) {
+    if (splits <= 1) return 0;
+    return ((splits * bh * sq * d * 4 + 255) & ~(size_t)255) + ((splits * bh * sq * 4 + 255) & ~(size_t)255);
+}
+
+size_t fv_sdpa_splitkv_choose(size_t bh, size_t sq, size_t sk) {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        return n;
+    }();
+    const size_t bm = (size_t)fv_internal_flash_block_m();
+    const size_t wgs = bh * ((sq + bm - 1) / bm), nkt = (sk + 63) / 64;
+    if (wgs == 0 || wgs >= (size_t)cus) return 1;               // the query tiles alone fill the CUs
+    // Cost model (microseconds, measured on MI355X): a workgroup costs about 10 fixed + 1.7 per 64-key
+    // tile, workgroups run in rounds of one per CU, and the merge reads `s` f32 partials at about
+    // 4 TB/s. Take the cheapest split count, if it wins by more than 10 %.
+    auto cost = [&](size_t sp) {
+        const size_t per = (nkt + sp - 1) / sp, real = (nkt + per - 1) / per;
+        const double rounds = (double)((wgs * real + cus - 1) / cus);
+        const double merge = real > 1 ? (double)(real * bh * sq) * 128.0 * 4.0 / 4.0e6 + 5.0 : 0.0;
+        return rounds * (10.0 + 1.7 * (double)per) + merge;
+    };
+    size_t best = 1;
+    double best_cost = cost(1);
+    for (size_t sp = 2; sp <= 16 && sp * 8 <= nkt; sp++) {        // at least 8 key tiles (4 phases) per split
+        const double c = cost(sp);
+        if (c < best_cost) best_cost = c, best = sp;
+    }
+    return best_cost < 0.9 * cost(1) ? best : 1;
+}
+
+int fv_sdpa_dense_bf16_splitkv(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
+                               int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
+                               size_t q_rows, size_t k_rows, size_t v_rows, size_t splits, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+    MaskArgs m;
+    m.q_rows = q_rows;
+    m.k_rows = k_rows;
+    m.v_rows = v_rows;
+    m.splits = splits ? splits : 1;
+    m.workspace = workspace;
+    m.workspace_bytes = workspace_bytes;
     return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, m, stream);
 }
 

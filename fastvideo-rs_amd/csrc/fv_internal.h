@@ -26,6 +26,12 @@ struct FlashParams {
     // elements between consecutive (batch, head) planes of q, k and v: s * d when contiguous, larger
     // when the operand is a row window of a longer plane (a KV cache read in place)
     long q_plane, k_plane, v_plane;
+    // Split-KV (dense launches only): kv_split > 1 gives every (head, query tile) kv_split workgroups,
+    // each walking split_tiles key tiles and writing its own normalised partial output (f32
+    // [split][bh][sq][d]) and base-2 log-sum-exp ([split][bh][sq]) for the merge kernel.
+    int kv_split, split_tiles;
+    float* part_o;
+    float* part_lse;
 };
 
 struct VsaFineParams {
@@ -70,6 +76,9 @@ extern "C" hipError_t fv_internal_launch_tile_qkv(const void* x, int x_is_bf16, 
 extern "C" int fv_internal_launch_composed_mfma(const float* q, const float* k, const float* v, const float* mask,
                                                 long mask_bh_stride, float* out, size_t bh, int sq, int sk, int d,
                                                 float scale, hipStream_t st);
+extern "C" hipError_t fv_internal_launch_splitkv_merge(const float* part_o, const float* part_lse, void* out,
+                                                       int out_is_bf16, size_t rows, int d, int splits,
+                                                       hipStream_t st);
 extern "C" hipError_t fv_internal_init_flash(void);
 extern "C" hipError_t fv_internal_init_vsa(void);
 extern "C" hipError_t fv_internal_launch_fine(const fv::VsaFineParams* p, hipStream_t st);

@@ -233,11 +233,23 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
         rc = fv_sdpa_vdn_window_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
                                      window->video_start, window->frame_tokens, window->frames, window->chunk,
                                      window->radius, st);
-    else if (q.strided() || k.strided() || v.strided())
-        rc = fv_sdpa_dense_bf16_strided(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
-                                        q.plane_rows, k.plane_rows, v.plane_rows, st);
-    else
-        rc = fv_sdpa_dense_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc, st);
+    else {
+        // few query tiles against many keys: split the keys over more workgroups (fv_sdpa_splitkv_choose)
+        const size_t splits = fv_sdpa_splitkv_choose(s->b * s->h, s->sq, s->sk);
+        Tensor ws;
+        if (splits > 1) {
+            auto rw = Tensor::alloc({fv_sdpa_splitkv_workspace_bytes(s->b * s->h, s->sq, s->d, splits) / 4}, DType::F32, st);
+            if (!is_ok(rw)) return std::get<TensorError>(rw);
+            ws = std::move(std::get<Tensor>(rw));
+            rc = fv_sdpa_dense_bf16_splitkv(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
+                                            q.plane_rows, k.plane_rows, v.plane_rows, splits, ws.data, ws.numel() * 4, st);
+        } else if (q.strided() || k.strided() || v.strided()) {
+            rc = fv_sdpa_dense_bf16_strided(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
+                                            q.plane_rows, k.plane_rows, v.plane_rows, st);
+        } else {
+            rc = fv_sdpa_dense_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc, st);
+        }
+    }
     if (rc == FV_DECLINED) return std::optional<Tensor>{};
     if (rc != FV_OK) return msg("sdpa: " + rc_message(rc));
     ((causal || window) ? g_causal : g_fused)++;

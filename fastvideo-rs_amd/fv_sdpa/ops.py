@@ -9,7 +9,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["sdpa_dense_bf16", "sdpa_dense_bf16_windows", "sdpa_block_causal_bf16", "sdpa_vdn_window_bf16", "cast_f32_bf16", "cast_bf16_f32", "sdpa_supported"]
+__all__ = ["sdpa_dense_bf16", "sdpa_dense_bf16_windows", "sdpa_dense_bf16_splitkv", "splitkv_choose", "sdpa_block_causal_bf16", "sdpa_vdn_window_bf16", "cast_f32_bf16", "cast_bf16_f32", "sdpa_supported"]
 
 
 def _stream():
@@ -69,6 +69,31 @@ def sdpa_dense_bf16_windows(q, k, v, scale=None, out_bf16=False):
     _lib.check(_lib.lib().fv_sdpa_dense_bf16_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                                      int(out_bf16), bh, sq, sk, d, scale, rows[0], rows[1], rows[2],
                                                      _stream()))
+    return out
+
+
+def splitkv_choose(bh, sq, sk):
+    """Key splits the library would use for this shape on the current device (1 = none)."""
+    return int(_lib.lib().fv_sdpa_splitkv_choose(bh, sq, sk))
+
+
+def sdpa_dense_bf16_splitkv(q, k, v, splits=None, scale=None, out_bf16=False):
+    """`sdpa_dense_bf16_windows` with the keys of every query tile split over `splits` workgroups
+    (default: the library's choice) and merged: for calls with few query tiles and many keys."""
+    rows = [_plane_rows(t, n) for t, n in ((q, "q"), (k, "k"), (v, "v"))]
+    bh, sq, d = q.shape
+    if k.shape != v.shape or k.shape[0] != bh or k.shape[2] != d:
+        raise ValueError(f"k/v {tuple(k.shape)}/{tuple(v.shape)} do not match q {tuple(q.shape)}")
+    sk = k.shape[1]
+    lib = _lib.lib()
+    splits = splitkv_choose(bh, sq, sk) if splits is None else int(splits)
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    out = torch.empty((bh, sq, d), device=q.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    nbytes = int(lib.fv_sdpa_splitkv_workspace_bytes(bh, sq, d, max(splits, 1)))
+    ws = torch.empty(max(nbytes, 256), device=q.device, dtype=torch.uint8)
+    _lib.check(lib.fv_sdpa_dense_bf16_splitkv(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), int(out_bf16), bh,
+                                              sq, sk, d, scale, rows[0], rows[1], rows[2], splits, ws.data_ptr(), nbytes,
+                                              _stream()))
     return out
 
 

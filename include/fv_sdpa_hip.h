@@ -60,6 +60,23 @@ int fv_sdpa_dense_bf16_strided(const uint16_t* q, const uint16_t* k, const uint1
                                int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                                size_t q_rows, size_t k_rows, size_t v_rows, void* stream);
 
+/* Split-KV form of the dense kernel for calls whose query tiles do not fill the GPU (a block of one
+ * latent frame against a long KV cache, a few prefix rows against the whole sequence): every
+ * (head, query tile) gets `splits` workgroups, each walking a contiguous share of the key tiles and
+ * writing a normalised f32 partial + its base-2 log-sum-exp into `workspace`; a merge kernel combines
+ * them into `out`. Same operands as fv_sdpa_dense_bf16_strided. No counterpart in the reference, whose
+ * kernels run one CTA per query tile (rt/attn.rs:378-395). fv_sdpa_splitkv_choose: the split count this
+ * library would pick for a shape on the current device (1 = none: use the plain entry; fv_rt_sdpa
+ * applies it by itself); splits is clamped so that no split is empty. workspace: 256-byte aligned,
+ * fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits) bytes. Results agree with the unsplit kernel
+ * to rounding (each split normalises by its own row sum before the merge). */
+size_t fv_sdpa_splitkv_choose(size_t bh, size_t sq, size_t sk);
+size_t fv_sdpa_splitkv_workspace_bytes(size_t bh, size_t sq, size_t d, size_t splits);
+int fv_sdpa_dense_bf16_splitkv(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
+                               int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
+                               size_t q_rows, size_t k_rows, size_t v_rows, size_t splits, void* workspace,
+                               size_t workspace_bytes, void* stream);
+
 /* rt/attn.rs:652-730 `device_mma_sdpa_causal` + kernels/attn2.cu:626-642
  * `flash_mma_fwd2_causal_d128`: the same under BlockCausal{block_tokens,
  * window, sink} (rt/attn.rs:441-453): query i sees key j iff
