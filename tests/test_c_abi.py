@@ -1,0 +1,27 @@
+"""The header is a plain C header and the library a plain C ABI: a C11 program (gcc -pedantic -Werror)
+includes include/fv_sdpa_hip.h, links libfv_sdpa_hip.so and calls host-only entry points. No GPU."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+from util import ROOT
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="no C compiler")
+def test_header_compiles_as_c_and_links(tmp_path):
+    pkg = os.path.join(ROOT, "fastvideo-rs_amd")
+    exe = str(tmp_path / "host_calls")
+    subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                           os.path.join(ROOT, "tests", "c_abi", "host_calls.c"), "-o", exe, "-L", pkg, "-lfv_sdpa_hip",
+                           "-Wl,-rpath," + pkg, "-Wl,-rpath,/opt/rocm/lib"])
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, (out.returncode, out.stdout, out.stderr)
+    line = out.stdout.strip()
+    assert "supported=10 " in line and "tiles=624 topk=125 " in line
+    assert "kvmove=30,30,60,0 " in line              # wan/causal.rs:901-906
+    assert "block_causal=1170,2,0 " in line          # rt/attn.rs:630-645: 3 frames of 390 tokens, window 6 frames = 2 blocks
+    assert "shards=0,6,6,5 " in line                 # rt/sp.rs:66-74
+    assert "backend=1 route=2:1,2 " in line
+    assert "local_attn_size=-1 keeps a 21-frame KV window" in line   # the refused plan's message
