@@ -43,21 +43,10 @@ struct TileGeo {
 typedef __attribute__((address_space(1))) void glb_void;
 typedef __attribute__((address_space(3))) void lds_void;
 
-// One wave-wide LDS-DMA instruction: lane i copies 16 B from its own global
-// address to LDS byte address lds_base + 16 i (lds_base wave-uniform). Issued as
-// inline asm so that the compiler's wait-count insertion does not serialise
-// later LDS reads of OTHER buffers behind it; the kernels order these loads with
-// wait_vmcnt<N>() + block_barrier() themselves.
-FV_DEV void lds_dma16(unsigned lds_base, const void* gptr) {
-    asm volatile(
-        "s_mov_b32 m0, %0\n\t"
-        "s_nop 0\n\t"
-        "global_load_lds_dwordx4 %1, off"
-        :
-        : "s"(lds_base), "v"(gptr)
-        : "memory");   // m0 is a reserved scratch register: the compiler sets it right before
-                       // each of its own uses and keeps nothing live in it across statements
-}
+// LDS-DMA: one wave-wide `global_load_lds_dwordx4` copies, per lane i, 16 B from the lane's global
+// address to LDS byte address lds_base + 16 i (lds_base wave-uniform, in m0). It is issued as inline
+// asm so that the compiler's wait-count insertion does not serialise later LDS reads of OTHER buffers
+// behind it; the kernels order these loads with wait_vmcnt<N>() + block_barrier() themselves.
 
 // Workgroup barrier without the memory fences of __syncthreads() (a fence
 // would wait for every outstanding LDS-DMA load, defeating the prefetch). LDS
@@ -87,7 +76,8 @@ FV_DEV void lds_dma16_s(unsigned lds_base, const void* sbase_in, unsigned voff) 
         "global_load_lds_dwordx4 %1, %2"
         :
         : "s"(lds_base), "v"(voff), "s"(sbase)
-        : "memory");
+        : "memory");   // m0 is a reserved scratch register: the compiler sets it right before each of
+                       // its own uses and keeps nothing live in it across statements
 }
 
 // Per-lane source offsets of the tile loads, computed once per kernel: a wave-wide
@@ -136,35 +126,6 @@ struct TileDma {
     static FV_DEV void issue_prepared(const Prepared& d, int it) {
         lds_dma16_s(d.lds + it * 1024, (const void*)d.base, d.off[it]);
     }
-    // The same without per-descriptor lane offsets (scalars only): the tail clamp, needed by
-    // the last key tile alone, is then taken at issue time behind a wave-uniform branch.
-    struct Target {
-        unsigned long long base;
-        unsigned lds;
-        int rows_valid;
-    };
-    FV_DEV Target target(lds_u8* buf, const uint16_t* tile_base, int rows_valid, int wave) const {
-        Target d;
-        d.base = (unsigned long long)tile_base;
-        d.lds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 1024);
-        d.rows_valid = rows_valid;
-        return d;
-    }
-    template <bool IS_V>
-    FV_DEV void issue_target(const Target& d) const {
-        if (d.rows_valid >= kTileRows) {
-#pragma unroll
-            for (int it = 0; it < ITER; it++)
-                lds_dma16_s(d.lds + it * 1024, (const void*)d.base, IS_V ? voff[it] : koff[it]);
-        } else {
-#pragma unroll
-            for (int it = 0; it < ITER; it++) {
-                const unsigned off = IS_V ? voff[it] : koff[it];
-                const int over = max(0, (int)(off / G::kRow) - (d.rows_valid - 1));
-                lds_dma16_s(d.lds + it * 1024, (const void*)d.base, off - over * G::kRow);
-            }
-        }
-    }
     // tile_base (wave-uniform) points at the tile's first row. Rows >= rows_valid
     // re-read the last valid row: the caller masks their scores to -inf, so their
     // content only has to be finite data the tensor already holds.
@@ -185,28 +146,6 @@ struct TileDma {
         }
     }
 };
-
-// Issue the asynchronous loads of one 64 x 128 bf16 tile whose rows are
-// contiguous in global memory (256 B apart). NW waves share the tile, 4 rows
-// per wave instruction. Rows >= rows_valid re-read the last valid row (the
-// caller masks their scores to -inf, so their content only has to be finite
-// data the tensor already holds). Completion is tracked by vmcnt: 16 / NW
-// instructions per wave and tile. This is the general (tail-safe) form; full
-// tiles go through TileDma::issue.
-template <int NW, bool IS_V>
-FV_DEV void tile_load_async(lds_u8* buf, const uint16_t* g, int rows_valid, int wave, int lane) {
-    constexpr int ITER = 16 / NW;
-    const int p = lane & 15;
-    const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 4 * kRowBytes);
-#pragma unroll
-    for (int it = 0; it < ITER; it++) {
-        const int R = (wave * ITER + it) * 4;
-        const int r = R + (lane >> 4);
-        const int c = IS_V ? (p ^ ((r & 3) << 2)) : (p ^ (r & 15));
-        const int rs = min(r, rows_valid - 1);
-        lds_dma16(base + it * 4 * kRowBytes, g + (size_t)rs * 128 + c * 8);
-    }
-}
 
 // Per-lane read bases into a swizzled tile.
 struct TileReadBases {

@@ -48,16 +48,6 @@ FV_DEV f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
-// Exchange between the two 32-lane halves of a wave: returns the value held by
-// lane l ^ 32.
-FV_DEV float other_half(float x) {
-    const unsigned u = __builtin_bit_cast(unsigned, x);
-    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    // r[0] = {lo, lo}, r[1] = {hi, hi}
-    const unsigned lo = r[0], hi = r[1];
-    return __builtin_bit_cast(float, (threadIdx.x & 32) ? lo : hi);
-}
-
 // max / sum over the pair of lanes {l, l ^ 32}, result in both.
 FV_DEV float pair_max(float x) {
     const unsigned u = __builtin_bit_cast(unsigned, x);
