@@ -207,3 +207,29 @@ def test_full_size_rows_of_ones(fv, bh, s):
     err = (out - 1.0).abs().max().item()
     print(f"max |out - 1| = {err:.3e}")
     assert err <= 4e-3     # P is rounded to bf16 (2^-9 relative) before it meets V; l sums the unrounded P
+
+
+@pytest.mark.parametrize("d", [128, 64])
+def test_extreme_score_ranges(fv, oracle, d):
+    """Nearly one-hot rows (scores of magnitude ~10^2: the running max jumps by far more than the lazy
+    rescale threshold, probabilities underflow to zero), uniform rows (q = 0: the plain mean of V) and
+    rows whose large scores are all equal."""
+    import torch
+
+    bh, sq, sk = 2, 300, 700
+    announce(f"dense extreme scores d={d}")
+    rng = np.random.Generator(np.random.PCG64(31))
+    q = oracle.quantize_bf16((rng.standard_normal((bh, sq, d)) * 6).astype(np.float32))
+    k = oracle.quantize_bf16((rng.standard_normal((bh, sk, d)) * 6).astype(np.float32))
+    v = oracle.quantize_bf16(rng.standard_normal((bh, sk, d)).astype(np.float32))
+    q[:, 10] = 0.0                        # uniform row
+    q[:, 11] = 4.0
+    k[0] = 8.0                            # head 0: every key identical -> all scores equal and large
+    got = fv.sdpa_dense_bf16(*(to_dev_bf16(x) for x in (q, k, v)))
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    want = oracle.sdpa_f64(q, k, v)
+    assert np.isfinite(got).all()
+    assert_parity(got, want, f"dense_extreme_d{d}", max_abs=2e-2)
+    assert np.abs(got[:, 10] - v.mean(axis=1)).max() < 2e-3
+    assert np.abs(got[0] - v[0].mean(axis=0)).max() < 2e-3
