@@ -103,9 +103,16 @@ static void transpose_one(const float* x, float* y, size_t r, size_t c) {
 void fvo_sdpa_composed(const float* q, const float* k, const float* v, const float* mask,
                        float* out, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                        int threads) {
-    float* kt = (float*)malloc(sizeof(float) * bh * d * sk);
-    float* scores = (float*)malloc(sizeof(float) * bh * sq * sk);
-    float* probs = (float*)malloc(sizeof(float) * bh * sq * sk);
+    /* calloc: sizes of zero stay valid, and the buffers start defined */
+    float* kt = (float*)calloc(bh * d * sk + 1, sizeof(float));
+    float* scores = (float*)calloc(bh * sq * sk + 1, sizeof(float));
+    float* probs = (float*)calloc(bh * sq * sk + 1, sizeof(float));
+    if (!kt || !scores || !probs) {
+        free(kt);
+        free(scores);
+        free(probs);
+        return;
+    }
     for (size_t b = 0; b < bh; b++) transpose_one(k + b * sk * d, kt + b * d * sk, sk, d);
     fvo_matmul(q, kt, scores, bh, sq, d, sk, threads);           /* q.matmul(k^T)   */
     for (size_t i = 0; i < bh * sq * sk; i++) scores[i] = scores[i] * scale; /* mul_scalar */
