@@ -45,6 +45,7 @@ SIGNATURES = {
     "fv_sdpa_block_causal_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float,
                                             _sz, _sz, _sz, _vp]),
     "fv_cast_f32_bf16": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "fv_softmax_last": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _vp]),
     "fv_cast_bf16_f32": (C.c_int, [_vp, _vp, _sz, _vp]),
     "fv_sdpa_composed_f32": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _vp, _sz, _sz, _sz, _sz, C.c_float, _vp]),
     "fv_sdpa_init": (C.c_int, []),

@@ -9,7 +9,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["sdpa_dense_bf16", "sdpa_dense_bf16_windows", "sdpa_dense_bf16_splitkv", "splitkv_choose", "sdpa_block_causal_bf16", "sdpa_vdn_window_bf16", "cast_f32_bf16", "cast_bf16_f32", "sdpa_supported"]
+__all__ = ["sdpa_dense_bf16", "sdpa_dense_bf16_windows", "sdpa_dense_bf16_splitkv", "splitkv_choose", "sdpa_block_causal_bf16", "sdpa_vdn_window_bf16", "cast_f32_bf16", "cast_bf16_f32", "softmax_last", "sdpa_supported"]
 
 
 def _stream():
@@ -129,3 +129,19 @@ def cast_bf16_f32(x):
     y = torch.empty(x.shape, device=x.device, dtype=torch.float32)
     _lib.check(_lib.lib().fv_cast_bf16_f32(x.data_ptr(), y.data_ptr(), x.numel(), _stream()))
     return y
+
+
+def softmax_last(x, out_bf16=False, out=None):
+    """Softmax over the trailing axis of an f32 tensor (rt/ops.rs:377-401 `softmax_last_device` /
+    `softmax_last_bf16_device`); `out=x` runs the f32 form in place."""
+    _need(x, torch.float32, "x")
+    width = x.shape[-1] if x.dim() else 1
+    rows = x.numel() // width if width else 0
+    if out is None:
+        out = torch.empty(x.shape, device=x.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    else:
+        _need(out, torch.bfloat16 if out_bf16 else torch.float32, "out")
+        if out.shape != x.shape:
+            raise ValueError("out: shape differs from x")
+    _lib.check(_lib.lib().fv_softmax_last(x.data_ptr(), out.data_ptr(), int(out_bf16), rows, width, _stream()))
+    return out

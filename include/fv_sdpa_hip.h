@@ -104,6 +104,13 @@ int fv_cast_f32_bf16(const float* x, uint16_t* y, size_t n, void* stream);
 /* bf16 bits -> f32 (exact widening), rt/tensor.rs `to_f32_act`. */
 int fv_cast_bf16_f32(const uint16_t* x, float* y, size_t n, void* stream);
 
+/* rt/ops.rs:377-401 `softmax_last_device` / `softmax_last_bf16_device` + kernels/core.cu:177-252
+ * (host form rt/ops.rs:2178-2193): softmax over the contiguous trailing axis of x [rows, width],
+ * out[r, j] = exp(x[r, j] - max_r) * (1 / sum_r); out f32 (may alias x) or bf16 bits (RNE). The step
+ * between the two GEMMs of the reference's materialised attention and VSA coarse stage; the fused
+ * kernels here never call it. */
+int fv_softmax_last(const float* x, void* out, int out_is_bf16, size_t rows, size_t width, void* stream);
+
 /* rt/sdpa.rs:328-342 `sdpa_composed` on the device: out = softmax(scale * q k^T + mask) v,
  * f32 operands [bh, s, d] and f32 out; mask NULL, or additive [sq, sk] shared by every bh
  * (mask_per_bh == 0), or [bh, sq, sk] (mask_per_bh != 0). The path for masked calls and for
