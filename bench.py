@@ -8,8 +8,9 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache|kvcache1|composed) are for the
-design notes; the driver's line is the default `self`.
+Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache|kvcache1|composed|
+softmax|machine) are for the design notes; the driver's line is the default `self`. `machine` measures the box, not
+the library: the rate of an MFMA-only loop at several launch lengths and of a plain copy.
 """
 import argparse
 import json
@@ -334,6 +335,113 @@ def bench_prep(args):
     print(json.dumps(rec), flush=True)
 
 
+def bench_softmax(args):
+    """Row softmax entry on score matrices of the shapes the reference materialises: VSA coarse scores
+    (12 x 624 rows of 624), a 4096-key chunk, rows of a whole 32760-key call."""
+    import torch
+
+    import fv_sdpa
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    shapes = []
+    for rows, width in ((12 * 624, 624), (12 * 4096, 4096), (12 * 2048, 8190), (4096, 32760)):
+        x = torch.randn((rows, width), device=dev)
+        for bf in (False, True):
+            out = fv_sdpa.softmax_last(x, out_bf16=bf)
+            for _ in range(args.warmup):
+                fv_sdpa.softmax_last(x, out_bf16=bf, out=out)
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(args.steps):
+                fv_sdpa.softmax_last(x, out_bf16=bf, out=out)
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b) / args.steps
+            nbytes = rows * width * (4 + (2 if bf else 4))
+            shapes.append({"rows": rows, "width": width, "out": "bf16" if bf else "f32", "us": round(ms * 1e3, 2),
+                           "GBps": round(nbytes / ms / 1e6, 1)})
+        del x, out
+    head = shapes[2]
+    rec = {
+        "metric": "row softmax GB/s (12*4096 rows x 4096, f32 out)", "value": head["GBps"], "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["us"] / 1e3, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "fv_softmax_last over f32 score matrices", "shapes": shapes},
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(head["GBps"] / PEAK_HBM_GBS, 4), "traffic": None},
+    }
+    print(json.dumps(rec), flush=True)
+
+
+def bench_machine(args):
+    """What this box gives a kernel with nothing in its way: an MFMA-only loop (bf16 32x32x16, register
+    operands, 2 waves per SIMD on every CU) at launch lengths from tens of microseconds to tens of
+    milliseconds, and a plain 1 GiB copy. The long launches show the clock the chip holds under matrix
+    load; their rate is the ceiling an MFMA-bound kernel sees here."""
+    import ctypes as C
+
+    import torch
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    path = os.path.join(ROOT, "fastvideo-rs_amd", "libfv_probes.so")
+    if not os.path.exists(path):
+        print(f"bench.py: {path} is not built (make -C fastvideo-rs_amd/csrc)", file=sys.stderr)
+        sys.exit(4)
+    lib = C.CDLL(path)
+    lib.fv_probe_mfma_bf16.restype = C.c_int
+    lib.fv_probe_mfma_bf16.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.c_void_p]
+    lib.fv_probe_copy_f32x4.restype = C.c_int
+    lib.fv_probe_copy_f32x4.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+    stream = torch.cuda.current_stream().cuda_stream
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    blocks = 2 * cus
+    sink = torch.empty(blocks * 256, device=dev)
+    flops = C.c_double()
+    mfma = []
+    for pattern in (0, 1):
+        for iters in (64, 1024, 8192, 65536, 262144):
+            for rep in range(3):    # the last repetition is the one reported
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                rc = lib.fv_probe_mfma_bf16(sink.data_ptr(), blocks, iters, pattern, C.byref(flops), stream)
+                b.record()
+                torch.cuda.synchronize()
+                if rc != 0:
+                    raise RuntimeError(f"fv_probe_mfma_bf16 rc={rc}")
+            ms = a.elapsed_time(b)
+            tf = flops.value / ms / 1e9
+            # 4 SIMDs per CU, one 32x32x16 MFMA (32768 FLOP) per 32 cycles per SIMD when the pipe never idles
+            mfma.append({"operands": "random" if pattern else "constant", "iters": iters, "ms": round(ms, 4),
+                         "TFLOPs": round(tf, 1), "implied_clock_GHz": round(tf * 1e12 / (cus * 4 * 1024) / 1e9, 3)})
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for rep in range(3):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        rc = lib.fv_probe_copy_f32x4(src.data_ptr(), dst.data_ptr(), n // 16, 16 * cus, stream)
+        b.record()
+        torch.cuda.synchronize()
+        if rc != 0:
+            raise RuntimeError(f"fv_probe_copy_f32x4 rc={rc}")
+    copy_ms = a.elapsed_time(b)
+    copy_gbs = 2.0 * n / copy_ms / 1e6
+    long_run = mfma[-1]
+    rec = {
+        "metric": "MFMA-only bf16 TFLOP/s sustained on this box, random operands (not a library kernel)", "value": long_run["TFLOPs"],
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": 1, "warmup": 2, "ms_per_step": long_run["ms"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "machine probe: v_mfma_f32_32x32x16_bf16 loop, 2 waves per SIMD; 1 GiB copy", "cus": cus,
+                   "mfma_only": mfma, "copy_1GiB": {"ms": round(copy_ms, 4), "GBps_read_plus_write": round(copy_gbs, 1)}},
+        "roofline": {"bound": "mfma", "achieved": long_run["TFLOPs"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(long_run["TFLOPs"] / PEAK_BF16_TFLOPS, 4), "traffic": None},
+    }
+    print(json.dumps(rec), flush=True)
+
+
 def visible_pairs(sq, sk, bt):
     if bt == 0:
         return sq * sk
@@ -395,7 +503,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "kvcache1", "composed"])
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "kvcache1", "composed", "softmax", "machine"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
@@ -425,6 +533,12 @@ def main():
         return
     if args.workload == "composed":
         bench_composed(args)
+        return
+    if args.workload == "softmax":
+        bench_softmax(args)
+        return
+    if args.workload == "machine":
+        bench_machine(args)
         return
     fv_sdpa.lib()
     dev = torch.device("cuda:0")
