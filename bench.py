@@ -416,6 +416,24 @@ def bench_machine(args):
             # 4 SIMDs per CU, one 32x32x16 MFMA (32768 FLOP) per 32 cycles per SIMD when the pipe never idles
             mfma.append({"operands": "random" if pattern else "constant", "iters": iters, "ms": round(ms, 4),
                          "TFLOPs": round(tf, 1), "implied_clock_GHz": round(tf * 1e12 / (cus * 4 * 1024) / 1e9, 3)})
+    # the block-sparse fine kernel's load pattern alone: 16 KB tiles through LDS-DMA, 4 workgroups per CU
+    lib.fv_probe_tile_dma.restype = C.c_int
+    lib.fv_probe_tile_dma.argtypes = [C.c_void_p, C.c_uint, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double), C.c_void_p]
+    tiles_buf = torch.zeros(2 << 30, dtype=torch.uint8, device=dev)
+    nbytes = C.c_double()
+    dma = []
+    for region_tiles in (64, 4096, 131072):
+        for rep in range(3):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            rc = lib.fv_probe_tile_dma(tiles_buf.data_ptr(), region_tiles, 4 * cus, 1000, None, C.byref(nbytes), stream)
+            b.record()
+            torch.cuda.synchronize()
+            if rc != 0:
+                raise RuntimeError(f"fv_probe_tile_dma rc={rc}")
+        ms = a.elapsed_time(b)
+        dma.append({"region_MiB": region_tiles * 16 // 1024, "ms": round(ms, 4), "TBps": round(nbytes.value / ms / 1e9, 2)})
+    del tiles_buf
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
     dst = torch.empty_like(src)
@@ -435,7 +453,7 @@ def bench_machine(args):
         "unit": "TFLOP/s", "n_gpus": 1, "steps": 1, "warmup": 2, "ms_per_step": long_run["ms"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "machine probe: v_mfma_f32_32x32x16_bf16 loop, 2 waves per SIMD; 1 GiB copy", "cus": cus,
-                   "mfma_only": mfma, "copy_1GiB": {"ms": round(copy_ms, 4), "GBps_read_plus_write": round(copy_gbs, 1)}},
+                   "mfma_only": mfma, "tile_dma_only": dma, "copy_1GiB": {"ms": round(copy_ms, 4), "GBps_read_plus_write": round(copy_gbs, 1)}},
         "roofline": {"bound": "mfma", "achieved": long_run["TFLOPs"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(long_run["TFLOPs"] / PEAK_BF16_TFLOPS, 4), "traffic": None},
     }

@@ -10,8 +10,17 @@
 // mantissa and exponent (2^-2 .. 2^0, the bit activity of N(0,1) data), which costs more power.
 //
 // fv_probe_copy_f32x4: out[i] = in[i] in 16-byte units, grid-stride: the HBM rate a plain stream gets.
+//
+// fv_probe_tile_dma: the load side of the block-sparse fine kernel alone. Workgroups of 2 waves with
+// two 16 KB LDS buffers (4 workgroups per CU, as that kernel) stream 64-row x 256-byte tiles through
+// global_load_lds_dwordx4, always one tile in flight behind the one being waited for, no arithmetic.
+// The tiles come from the first `region_tiles` tiles of the source in a scattered order, so a small
+// region measures the L2 -> LDS path and a large one the path from HBM.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include "../fv_common.h"
+#include "../attn_core.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
@@ -98,9 +107,48 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const f32x4* __restrict
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) out[i] = in[i];
 }
 
+__global__ __launch_bounds__(128, 2) void probe_tile_dma_kernel(const uint16_t* src, unsigned region_tiles, int iters,
+                                                                float* sink) {
+    using namespace fv;
+    extern __shared__ __attribute__((aligned(16))) unsigned char probe_smem[];
+    lds_u8* kbuf = (lds_u8*)probe_smem;
+    lds_u8* vbuf = kbuf + kTileBytes;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    TileDma<2, 128> dma;
+    dma.init(wave, lane);
+    unsigned t = (blockIdx.x * 2654435761u) % region_tiles;
+    const unsigned step = 40503u % region_tiles + 1u;
+    dma.template issue<false>(kbuf, src + (size_t)t * kTileRows * 128, kTileRows, wave);
+#pragma unroll 1
+    for (int i = 0; i < iters; i++) {
+        t = (t + step) % region_tiles;
+        dma.template issue<true>(vbuf, src + (size_t)t * kTileRows * 128, kTileRows, wave);
+        wait_vmcnt<8>();    // the K tile landed; the V tile is in flight
+        t = (t + step) % region_tiles;
+        dma.template issue<false>(kbuf, src + (size_t)t * kTileRows * 128, kTileRows, wave);
+        wait_vmcnt<8>();    // the V tile landed
+    }
+    wait_vmcnt<0>();
+    __syncthreads();
+    if (sink) sink[(size_t)blockIdx.x * 128 + tid] = (float)kbuf[16 * tid] + (float)vbuf[16 * tid];
+}
+
 }  // namespace
 
 extern "C" {
+
+// `blocks` workgroups, each streaming 2 * iters + 1 tiles of 16 KB out of the first region_tiles tiles
+// of src (region_tiles * 16 KB readable bytes). Returns the bytes loaded through *bytes.
+int fv_probe_tile_dma(const void* src, unsigned region_tiles, int blocks, int iters, float* sink, double* bytes,
+                      void* stream) {
+    if (!src || region_tiles == 0 || blocks <= 0 || iters <= 0) return -(int)hipErrorInvalidValue;
+    if (((uintptr_t)src & 15) != 0) return -(int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(probe_tile_dma_kernel, dim3((unsigned)blocks), dim3(128), 40 * 1024 /* 4 workgroups per CU */, (hipStream_t)stream,
+                       (const uint16_t*)src, region_tiles, iters, sink);
+    if (bytes) *bytes = (double)fv::kTileBytes * (2.0 * iters + 1.0) * (double)blocks;
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? 0 : -(int)e;
+}
 
 // Launches `blocks` workgroups of 4 waves, each wave issuing 16 * iters MFMAs (32768 FLOP each).
 // `sink` holds blocks * 256 floats; pattern 0 = constant operands, 1 = random. Returns the FLOP count of the launch through *flops, 0 or a
