@@ -524,6 +524,9 @@ def main():
     ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "kvcache1", "composed", "softmax", "machine"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
+    ap.add_argument("--inputs", default="randn", choices=["randn", "zeros"],
+                    help="attention workloads only. zeros: the same launches on all-zero Q/K/V, a power experiment "
+                         "(same instruction stream, no bit activity in the operands); never the headline")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also launch one plain device copy of this many MiB (known HBM traffic, to scale "
                          "profiler byte counters); not part of the timed region")
@@ -567,6 +570,8 @@ def main():
     q = torch.randn((h, sq, d), generator=g, device=dev).to(torch.bfloat16)
     k = torch.randn((h, sk, d), generator=g, device=dev).to(torch.bfloat16)
     v = torch.randn((h, sk, d), generator=g, device=dev).to(torch.bfloat16)
+    if args.inputs == "zeros":
+        q.zero_(), k.zero_(), v.zero_()
     out = torch.empty((h, sq, d), device=dev, dtype=torch.bfloat16 if args.out_bf16 else torch.float32)
     lib = fv_sdpa.lib()
     stream = torch.cuda.current_stream().cuda_stream
@@ -627,7 +632,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic",
+        "data": "synthetic" if args.inputs == "randn" else "all-zero operands (power experiment, not a benchmark)",
         "config": {"workload": desc, "H": h, "Sq": sq, "Sk": sk, "d": d, "block_tokens": bt,
                    "out": "bf16" if args.out_bf16 else "f32", "flops_per_call": flops,
                    "dense_equivalent_flops": flops_dense_equiv},
