@@ -85,6 +85,32 @@ def test_every_tile_count_parity_and_key_tail(fv, oracle, sk, d):
         assert_parity(got.cpu().numpy(), want, f"dense_sweep_{sq}x{sk}")
 
 
+@pytest.mark.parametrize("bh,sq,sk,d", [(1100, 70, 200, 128), (300, 600, 130, 128), (600, 257, 65, 64), (520, 256, 64, 128)])
+def test_many_short_items(fv, oracle, bh, sq, sk, d):
+    """Launches of several rounds of short items (many heads, cross-attention-sized key sets): parity
+    against the oracle on a sample of heads (first and last workgroups included), and bit-identity
+    with the same heads computed in smaller calls (a head's result may not depend on what else the
+    launch holds or on where its workgroup runs)."""
+    import torch
+
+    announce(f"dense many items bh={bh} sq={sq} sk={sk} d={d}")
+    q, k, v = qkv(9100 + bh + sk, bh, sq, sk, d, 1.0)
+    qd, kd, vd = (to_dev_bf16(x) for x in (q, k, v))
+    got = fv.sdpa_dense_bf16(qd, kd, vd, out_bf16=False)
+    torch.cuda.synchronize()
+    heads = np.r_[0:3, bh // 2, bh - 3:bh]       # the oracle on a sample of heads, first and last items included
+    want = oracle.sdpa_composed(q[heads], k[heads], v[heads])
+    assert_parity(got[torch.from_numpy(heads).cuda()].cpu().numpy(), want, f"dense_many_items_{bh}x{sq}x{sk}")
+    step = max(1, 400 // ((sq + 255) // 256))    # heads per small call
+    for lo in range(0, bh, step):
+        hi = min(bh, lo + step)
+        part = fv.sdpa_dense_bf16(qd[lo:hi].contiguous(), kd[lo:hi].contiguous(), vd[lo:hi].contiguous(), out_bf16=False)
+        assert torch.equal(part, got[lo:hi]), f"heads {lo}..{hi} differ between the large and the small launch"
+    got16 = fv.sdpa_dense_bf16(qd, kd, vd, out_bf16=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(got16.float().cpu().numpy(), oracle.quantize_bf16(got.cpu().numpy()))
+
+
 def test_dense_vs_unrounded_f32_inputs(fv, oracle):
     import torch
 

@@ -44,6 +44,29 @@ def test_every_split_count_matches_the_unsplit_kernel(fv, oracle, bh, sq, sk, d)
     assert (got16.float() - base).abs().max().item() <= 2e-2
 
 
+def test_many_split_items(fv, oracle):
+    """40 heads x 2 query tiles x 8 splits = 640 workgroups of 4 key tiles (several rounds of short
+    items), against the unsplit kernel, the oracle, and the same heads in smaller calls."""
+    import torch
+
+    bh, sq, sk, d = 40, 300, 2000, 128
+    announce(f"splitkv many items bh={bh} sq={sq} sk={sk}")
+    q, k, v = qkv(4242, bh, sq, sk, d)
+    tq, tk, tv = (to_dev_bf16(x) for x in (q, k, v))
+    got = fv.sdpa_dense_bf16_splitkv(tq, tk, tv, splits=8)
+    base = fv.sdpa_dense_bf16(tq, tk, tv)
+    torch.cuda.synchronize()
+    assert (got - base).abs().max().item() <= 2e-3
+    heads = np.array([0, 1, 20, 38, 39])
+    assert_parity(got[torch.from_numpy(heads).cuda()].cpu().numpy(), oracle.sdpa_composed(q[heads], k[heads], v[heads]),
+                  "splitkv_many_items")
+    # the same heads in smaller calls: bit-identical partials and merge
+    for lo in range(0, bh, 10):
+        part = fv.sdpa_dense_bf16_splitkv(tq[lo:lo + 10].contiguous(), tk[lo:lo + 10].contiguous(),
+                                          tv[lo:lo + 10].contiguous(), splits=8)
+        assert torch.equal(part, got[lo:lo + 10])
+
+
 def test_choice_and_windows(fv, oracle):
     import torch
 
