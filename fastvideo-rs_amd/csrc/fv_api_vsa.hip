@@ -287,26 +287,10 @@ static int vsa_attention_common(const void* q, const void* k, const void* v, int
     float* coarse = (float*)(ws + w.coarse);
     uint32_t* sel = selected_out ? selected_out : (uint32_t*)(ws + w.selected);
     const uint16_t *qt = (const uint16_t*)q, *kt = (const uint16_t*)k, *vt = (const uint16_t*)v;
-    // tile-ordered input: identity slot map (null), rows per bh = padded
-    const int32_t* mean_map = tiled ? nullptr : slot_src;
-    const size_t mean_rows = tiled ? padded : seq;
-    const int in16 = tiled ? 1 : qkv_is_bf16;
     hipStream_t st = (hipStream_t)stream;
     hipError_t e;
     int rc;
-    // 1. tile means (rt/vsa.rs:378-384)
-    for (int i = 0; i < 3; i++) {
-        const void* x = i == 0 ? q : (i == 1 ? k : v);
-        float* m = i == 0 ? qc : (i == 1 ? kc : vc);
-        e = fv_internal_launch_tile_mean(x, in16, mean_map, block_sizes, m, bh, mean_rows, (int)dim, (int)num_tiles,
-                                         0, st);
-        if (e != hipSuccess) return fv_fail_hip(e, "vsa_tile_mean");
-    }
-    // 2. coarse attention over tiles; raw scores kept for the selection (rt/vsa.rs:385-394)
-    if ((rc = fv_vsa_coarse(qc, kc, vc, scores, coarse, bh, num_tiles, dim, scale, stream))) return rc;
-    // 3. top-k tiles per query tile (rt/vsa.rs:398-400)
-    if ((rc = fv_vsa_topk(scores, sel, bh * num_tiles, num_tiles, topk, stream))) return rc;
-    // 4. fine stage on tile-ordered bf16 copies (rt/vsa.rs:406-414)
+    // 4 (moved up). tile-ordered bf16 copies for the fine stage (rt/vsa.rs:406-414)
     if (!tiled) {
         uint16_t* tq = (uint16_t*)(ws + w.qt);
         uint16_t* tk = (uint16_t*)(ws + w.kt);
@@ -316,6 +300,22 @@ static int vsa_attention_common(const void* q, const void* k, const void* v, int
         if ((rc = fv_vsa_tile_qkv(v, qkv_is_bf16, slot_src, tv, bh, seq, padded, dim, stream))) return rc;
         qt = tq, kt = tk, vt = tv;
     }
+    // 1. tile means (rt/vsa.rs:378-384). Of bf16 operands they are taken from the tile-ordered copies
+    //    (the same values in the same slot order, read as contiguous rows: half the time of the gather
+    //    from token order); f32 operands are pooled unrounded, so they are read where they lie.
+    const bool from_tiles = tiled || qkv_is_bf16;
+    for (int i = 0; i < 3; i++) {
+        const void* x = from_tiles ? (const void*)(i == 0 ? qt : (i == 1 ? kt : vt)) : (i == 0 ? q : (i == 1 ? k : v));
+        float* m = i == 0 ? qc : (i == 1 ? kc : vc);
+        // tile-ordered input: identity slot map (null), rows per bh = padded
+        e = fv_internal_launch_tile_mean(x, from_tiles ? 1 : 0, from_tiles ? nullptr : slot_src, block_sizes, m, bh,
+                                         from_tiles ? padded : seq, (int)dim, (int)num_tiles, 0, st);
+        if (e != hipSuccess) return fv_fail_hip(e, "vsa_tile_mean");
+    }
+    // 2. coarse attention over tiles; raw scores kept for the selection (rt/vsa.rs:385-394)
+    if ((rc = fv_vsa_coarse(qc, kc, vc, scores, coarse, bh, num_tiles, dim, scale, stream))) return rc;
+    // 3. top-k tiles per query tile (rt/vsa.rs:398-400)
+    if ((rc = fv_vsa_topk(scores, sel, bh * num_tiles, num_tiles, topk, stream))) return rc;
     // 5. out = coarse * gate + sparse, back in token order: fused into the fine kernel's epilogue
     //    (no f32 sparse buffer: 2 x 200 MB of traffic and 200 MB of workspace less at Wan 480p)
     fv::VsaFineParams p;
