@@ -128,20 +128,22 @@ constexpr int kCoarseRows = 8;
 __global__ __launch_bounds__(256) void vsa_coarse_pv_kernel(
     const float* __restrict__ scores, const float* __restrict__ vc, float* __restrict__ coarse,
     int nb) {
-    extern __shared__ float p_lds[];   // [kCoarseRows][nb]
+    extern __shared__ __attribute__((aligned(16))) float p_lds[];   // [kCoarseRows][nbp], rows 16-byte aligned
     __shared__ float red[kCoarseRows][4];
     __shared__ float stat[kCoarseRows];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int q0 = blockIdx.x * kCoarseRows;
     const long bh = blockIdx.y;
     const int rows = min(kCoarseRows, nb - q0);
+    const int nbp = (nb + 3) & ~3;
     const float* sb = scores + (bh * nb + q0) * (long)nb;
-    for (int e = tid; e < rows * nb; e += 256) p_lds[e] = sb[e];
+    for (int r = 0; r < rows; r++)
+        for (int j = tid; j < nb; j += 256) p_lds[r * nbp + j] = sb[(long)r * nb + j];
     __syncthreads();
     // row max
     for (int r = 0; r < rows; r++) {
         float m = neg_inf();
-        for (int j = tid; j < nb; j += 256) m = fmaxf(m, p_lds[r * nb + j]);
+        for (int j = tid; j < nb; j += 256) m = fmaxf(m, p_lds[r * nbp + j]);
         for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
         if (lane == 0) red[r][wave] = m;
     }
@@ -152,8 +154,8 @@ __global__ __launch_bounds__(256) void vsa_coarse_pv_kernel(
         const float m = stat[r];
         float s = 0.f;
         for (int j = tid; j < nb; j += 256) {
-            const float e = expf(p_lds[r * nb + j] - m);
-            p_lds[r * nb + j] = e;
+            const float e = expf(p_lds[r * nbp + j] - m);
+            p_lds[r * nbp + j] = e;
             s += e;
         }
         for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
@@ -162,12 +164,12 @@ __global__ __launch_bounds__(256) void vsa_coarse_pv_kernel(
     __syncthreads();
     if (tid < rows) stat[tid] = 1.0f / (red[tid][0] + red[tid][1] + red[tid][2] + red[tid][3]);
     __syncthreads();
-    // each half-block owns four rows; lane d accumulates over all key tiles, four vc rows
-    // in flight per step
+    // each half-block owns four rows; lane d accumulates over all key tiles in ascending order, four
+    // vc rows in flight per step and the four weights of a row in one 16-byte LDS read
     constexpr int kOwn = kCoarseRows / 2;
     const int d = tid & 127, rh = tid >> 7;
     const float* vb = vc + bh * nb * 128L + d;
-    const float* pr = p_lds + (kOwn * rh) * nb;
+    const float* pr = p_lds + (kOwn * rh) * nbp;
     float a[kOwn];
 #pragma unroll
     for (int r = 0; r < kOwn; r++) a[r] = 0.f;
@@ -177,14 +179,16 @@ __global__ __launch_bounds__(256) void vsa_coarse_pv_kernel(
 #pragma unroll
         for (int u = 0; u < 4; u++) vv[u] = vb[(long)(kt + u) * 128];
 #pragma unroll
-        for (int u = 0; u < 4; u++)
+        for (int r = 0; r < kOwn; r++) {
+            const f32x4 p4 = *reinterpret_cast<const f32x4*>(pr + r * nbp + kt);
 #pragma unroll
-            for (int r = 0; r < kOwn; r++) a[r] += pr[r * nb + kt + u] * vv[u];
+            for (int u = 0; u < 4; u++) a[r] += p4[u] * vv[u];
+        }
     }
     for (; kt < nb; kt++) {
         const float vv = vb[(long)kt * 128];
 #pragma unroll
-        for (int r = 0; r < kOwn; r++) a[r] += pr[r * nb + kt] * vv;
+        for (int r = 0; r < kOwn; r++) a[r] += pr[r * nbp + kt] * vv;
     }
 #pragma unroll
     for (int r = 0; r < kOwn; r++)
@@ -557,7 +561,7 @@ extern "C" hipError_t fv_internal_launch_coarse(const float* qc, const float* kc
     hipLaunchKernelGGL(vsa_coarse_scores_kernel, g1, dim3(256), 0, st, qc, kc, scores, nb, dim, scale);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || !coarse) return e;
-    const size_t lds = sizeof(float) * kCoarseRows * (size_t)nb;
+    const size_t lds = sizeof(float) * kCoarseRows * (size_t)((nb + 3) & ~3);
     e = fv_internal_init_vsa();
     if (e != hipSuccess) return e;
     const dim3 g2((nb + kCoarseRows - 1) / kCoarseRows, (unsigned)bh);
