@@ -129,6 +129,12 @@ struct TileDma {
     // tile_base (wave-uniform) points at the tile's first row. Rows >= rows_valid
     // re-read the last valid row: the caller masks their scores to -inf, so their
     // content only has to be finite data the tensor already holds.
+    // one of the ITER instructions of a full tile's load
+    template <bool IS_V>
+    FV_DEV void issue_one(lds_u8* buf, const uint16_t* tile_base, int wave, int it) const {
+        const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 1024);
+        lds_dma16_s(base + it * 1024, tile_base, IS_V ? voff[it] : koff[it]);
+    }
     template <bool IS_V>
     FV_DEV void issue(lds_u8* buf, const uint16_t* tile_base, int rows_valid, int wave) const {
         const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)buf + wave * ITER * 1024);
@@ -182,6 +188,24 @@ FV_DEV void qk_tile(const lds_u8* kb, int k_base, const bf16x8 (&qf)[8], f32x16 
     }
 }
 
+// qk_tile with `side(g)` after MFMA g (0..15): side work that rides under the matrix pipe.
+template <class Side>
+FV_DEV void qk_tile_side(const lds_u8* kb, int k_base, const bf16x8 (&qf)[8], f32x16 (&s)[2], Side&& side) {
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[b][i] = 0.f;
+#pragma unroll
+        for (int dk = 0; dk < 8; dk++) {
+            const bf16x8 a = lds_read_b128(kb + (k_base ^ (dk << 5)) + b * 32 * kRowBytes);
+            s[b] = mfma32(a, qf[dk], s[b]);
+            __builtin_amdgcn_sched_barrier(0);
+            side(b * 8 + dk);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
 // Online-softmax state of one query (replicated in lanes l and l^32; l_acc is
 // the lane's own share of the row sum).
 struct SoftmaxState {
@@ -198,8 +222,11 @@ constexpr float kRescaleLog2 = 6.0f;
 
 // Row max, lazy rescale of (l, O), P = 2^(s*sl2 - offset), bf16 pack.
 // pb[t] is the B operand (16 key slots x 32 queries) for key group t.
-FV_DEV void softmax_tile(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float sl2,
-                         bf16x8 (&pb)[4]) {
+// `side(part)` runs after the rescale (part 0) and after each 32-key half of the exponentials
+// (parts 1, 2): slots for side work, such as tile DMA issue, spread through the VALU stream.
+template <class Side>
+FV_DEV void softmax_tile_side(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float sl2,
+                              bf16x8 (&pb)[4], Side&& side) {
     const float NEG = neg_inf();
     float mx = s[0][0];
 #pragma unroll
@@ -221,6 +248,7 @@ FV_DEV void softmax_tile(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float
         st.m_used = st.m_run;
         st.ms_used = ms_new;
     }
+    side(0);
 #pragma unroll
     for (int b = 0; b < 2; b++) {
         f32x16 e;
@@ -236,7 +264,12 @@ FV_DEV void softmax_tile(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float
             for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
             pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
         }
+        side(1 + b);
     }
+}
+FV_DEV void softmax_tile(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float sl2,
+                         bf16x8 (&pb)[4]) {
+    softmax_tile_side(s, st, o, sl2, pb, [](int) {});
 }
 
 // softmax_tile over a pair of tiles (128 keys) with one shared max / rescale decision.

@@ -399,13 +399,18 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
     for (int i = 0; i < topk; i++) {
         wait_vmcnt<0>();     // K(i) landed
         block_barrier();     // ... for every wave; PV(i-1) finished everywhere: V buffer free
-        dma.template issue<true>(vbuf, vb + (size_t)tile * kTileElems * 128, kTileElems, wave);
         const int tile_nn = tile_at(i + 2);          // consumed an iteration from now
         f32x16 s[2];
-        qk_tile(kbuf, rb.k, qf, s);
+        // the 8 DMA instructions of V(i) go out one behind every second MFMA of QK(i), those of K(i+1)
+        // in three groups through the softmax: issued in one burst they hold the wave (in-order issue)
+        // while the CU's address path drains, 4 % of the kernel's time
+        const uint16_t* vsrc = vb + (size_t)tile * kTileElems * 128;
+        qk_tile_side(kbuf, rb.k, qf, s, [&](int g) {
+            if (g & 1) dma.template issue_one<true>(vbuf, vsrc, wave, g >> 1);
+        });
         block_barrier();     // K buffer free
         const bool more = i + 1 < topk;
-        if (more) dma.template issue<false>(kbuf, kb + (size_t)tile_next * kTileElems * 128, kTileElems, wave);
+        const uint16_t* ksrc = kb + (size_t)tile_next * kTileElems * 128;
         if (valid < kTileElems) {
 #pragma unroll
             for (int b = 0; b < 2; b++)
@@ -416,7 +421,13 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
                 }
         }
         bf16x8 pb[4];
-        softmax_tile(s, st, o, sl2, pb);
+        softmax_tile_side(s, st, o, sl2, pb, [&](int part) {
+            if (more) {
+                const int first = 3 * part, last = part == 2 ? 8 : first + 3;
+#pragma unroll
+                for (int it = first; it < last; it++) dma.template issue_one<false>(kbuf, ksrc, wave, it);
+            }
+        });
         if (more) wait_vmcnt<8>(); else wait_vmcnt<0>();   // V(i) landed; K(i+1) may be in flight
         block_barrier();
         pv_tile(vbuf, rb.v, pb, o);
