@@ -229,6 +229,18 @@ Result<bool> CausalKvCache::advance(size_t current_start, size_t n, size_t sink_
     return true;
 }
 
+Result<CausalKvCache::BlockKey> CausalKvCache::block_key(size_t current_start, size_t n, size_t sink_target) const {
+    std::lock_guard<std::mutex> g(mu_);
+    KvPointers p{0, 0, 0, false};
+    if (!layers_.empty()) p = KvPointers{layers_[0].global_end, layers_[0].local_end, layers_[0].sink_at, layers_[0].raw_valid};
+    auto mv = kv_plan(spec, p.global_end, p.local_end, current_start, n);
+    if (!is_ok(mv)) return std::get<TensorError>(mv);
+    const bool rebase = spec.rebase_sink && spec.sink > 0 && sink_target > 0 && p.sink_at != sink_target &&
+                        p.local_end >= spec.sink;
+    return BlockKey{p.local_end, current_start + n > p.global_end, std::get<KvMove>(mv).evicted, rebase,
+                    rebase && !p.raw_valid};
+}
+
 size_t CausalKvCache::bytes() const {
     std::lock_guard<std::mutex> g(mu_);
     size_t n = 0;
@@ -425,6 +437,15 @@ int fv_kv_cache_advance(fv_kv_cache* c, size_t current_start, size_t n, size_t s
     if (!c) return fv_invalid("kv cache: null argument");
     auto r = c->cache.advance(current_start, n, sink_target);
     if (!fv::rt::is_ok(r)) return fv_invalid(std::get<fv::rt::TensorError>(r).message.c_str());
+    return FV_OK;
+}
+
+int fv_kv_cache_block_key(const fv_kv_cache* c, size_t current_start, size_t n, size_t sink_target, size_t out5[5]) {
+    if (!c || !out5) return fv_invalid("kv cache: null argument");
+    auto r = c->cache.block_key(current_start, n, sink_target);
+    if (!fv::rt::is_ok(r)) return fv_invalid(std::get<fv::rt::TensorError>(r).message.c_str());
+    const auto& k = std::get<fv::rt::CausalKvCache::BlockKey>(r);
+    out5[0] = k.local_end, out5[1] = k.appends, out5[2] = k.evicted, out5[3] = k.rebase, out5[4] = k.take_raw;
     return FV_OK;
 }
 

@@ -96,6 +96,17 @@ class CausalKvCache {
     // current_start (sink target frame `sink_target`, 0: none) without its device work: what a graph
     // replay of that forward leaves behind.
     Result<bool> advance(size_t current_start, size_t n, size_t sink_target);
+    // wan/causal.rs:477-502 `block_key`: what a forward of n tokens at current_start (sink target frame
+    // `sink_target`, 0: none) does to the cache, from layer 0's pointers (every layer moves in step).
+    // Forwards with equal keys launch the same device work, so a captured graph of one serves the others.
+    struct BlockKey {
+        size_t local_end;
+        bool appends;       // the block extends the cache (false: an in-place re-run of cached frames)
+        size_t evicted;
+        bool rebase;        // the rebased-sink policy re-ropes the sink before this block
+        bool take_raw;      // ... and first takes the un-roped copy
+    };
+    Result<BlockKey> block_key(size_t current_start, size_t n, size_t sink_target) const;
     size_t bytes() const;
     const KvSpec spec;
 

@@ -35,6 +35,7 @@ SIGNATURES = {
     "fv_kv_cache_rebase_sink": (C.c_int, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "fv_kv_cache_set_pointers": (C.c_int, [_vp, _vp, _sz]),
     "fv_kv_cache_advance": (C.c_int, [_vp, _sz, _sz, _sz]),
+    "fv_kv_cache_block_key": (C.c_int, [_vp, _sz, _sz, _sz, _vp]),
     "fv_rope_bhsd": (C.c_int, [_vp, C.c_int, _sz, _vp, _vp, C.c_int, _vp, C.c_int, _sz, _sz, _sz, _sz, _vp]),
     "fv_kv_cache_free": (None, [_vp]),
     "fv_kv_cache_reset": (None, [_vp]),

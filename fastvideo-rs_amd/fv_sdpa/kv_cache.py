@@ -3,6 +3,7 @@
 layer. The windows `update` returns are torch views of the layer's persistent buffers (no copy);
 `sdpa(q, kw, vw, Plan.kv_window())` reads them in place.
 """
+import collections
 import ctypes as C
 
 import torch
@@ -10,7 +11,7 @@ import torch
 from . import _lib
 from .sdpa import TensorError, _desc, _FvTensor
 
-__all__ = ["KvSpec", "KvMove", "KvRope", "CausalKvCache", "kv_copy_tokens", "kv_shift_tokens_down", "rope_bhsd"]
+__all__ = ["KvSpec", "KvMove", "KvBlockKey", "KvRope", "CausalKvCache", "kv_copy_tokens", "kv_shift_tokens_down", "rope_bhsd"]
 
 
 class KvMove:
@@ -21,6 +22,10 @@ class KvMove:
 
     def __repr__(self):
         return f"KvMove(evicted={self.evicted}, local=[{self.local_start}, {self.local_end}), window_start={self.window_start})"
+
+
+class KvBlockKey(collections.namedtuple("KvBlockKey", "local_end appends evicted rebase take_raw")):
+    """wan/causal.rs:365-378: what a block forward does to the cache; equal keys, equal device work."""
 
 
 class KvRope:
@@ -151,6 +156,15 @@ class CausalKvCache:
         lib = _lib.lib()
         if lib.fv_kv_cache_advance(self._h, current_start, n, sink_target) != 0:
             raise TensorError(lib.fv_sdpa_last_error().decode())
+
+    def block_key(self, current_start, n, sink_target=0):
+        """wan/causal.rs:477-502: (local_end, appends, evicted, rebase, take_raw) of a forward of n tokens at
+        current_start; forwards with equal keys launch the same device work."""
+        out = (C.c_size_t * 5)()
+        lib = _lib.lib()
+        if lib.fv_kv_cache_block_key(self._h, current_start, n, sink_target, out) != 0:
+            raise TensorError(lib.fv_sdpa_last_error().decode())
+        return KvBlockKey(int(out[0]), bool(out[1]), int(out[2]), bool(out[3]), bool(out[4]))
 
     def rebase_sink(self, target, orig, new):
         """wan/causal.rs:733-776: re-rope every layer's sink keys to start at frame `target`;

@@ -218,6 +218,10 @@ int fv_kv_cache_set_pointers(fv_kv_cache* c, const size_t* in4, size_t layers);
 /* wan/causal.rs:503-536 `advance`: the host bookkeeping of one block forward of n tokens at current_start
  * (rebased-sink target frame sink_target, 0: none) on every layer, without its device work. */
 int fv_kv_cache_advance(fv_kv_cache* c, size_t current_start, size_t n, size_t sink_target);
+/* wan/causal.rs:477-502 `block_key`: out5 = {local_end, appends, evicted, rebase, take_raw} of a forward of
+ * n tokens at current_start (from layer 0's pointers): forwards with equal keys launch the same device
+ * work, so a captured graph of one serves the others. Errors as fv_kv_plan. */
+int fv_kv_cache_block_key(const fv_kv_cache* c, size_t current_start, size_t n, size_t sink_target, size_t out5[5]);
 /* wan/causal.rs:733-776 `rebase_sink` (static mode): re-rope every layer's sink keys to start at frame
  * `target`. orig_cos / orig_sin: tables of the sink's own frames (used once, to take the un-roped f32
  * copy by rotating back); new_cos / new_sin: tables of frames [target, target + sink): f32

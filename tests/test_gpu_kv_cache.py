@@ -328,3 +328,40 @@ def test_rebased_sink_policy_equals_the_oracles(fv, oracle, bf16):
         plain.rebase_sink(1, (dev(cos_o), dev(sin_o)), (dev(cos_o), dev(sin_o)))
     with pytest.raises(fv.TensorError, match="advance over an unwritten cache"):
         plain.advance(0, n)
+
+
+def test_block_keys_settle_once_the_window_is_full(fv):
+    """The reference's known answers for `block_key` (causal.rs:1196-1232; head dim 8 here instead of 2,
+    the rope kernel rotates 8 elements per thread): keys follow the fill — appends while the window fills, the first roll
+    takes the un-roped sink, then every block has the same key; an in-place re-run of a block neither
+    appends, rebases nor evicts."""
+    import torch
+
+    spec = fv.KvSpec.rolling_window(10, 6, 2, fv.KvRope.REBASED_SINK)
+    cache = fv.CausalKvCache(spec, 1)
+    blk = lambda start: (start + torch.arange(160, dtype=torch.float32, device="cuda")).reshape(1, 1, 20, 8)  # noqa: E731
+    tab = torch.ones((20, 8), device="cuda")
+    zero = torch.zeros((20, 8), device="cuda")
+    keys = []
+    for b in range(6):
+        start = b * 20
+        target = spec.sink_target(b * 2 + 2)
+        key = cache.block_key(start, 20, target)
+        keys.append(key)
+        if key.rebase:
+            cache.rebase_sink(target, (tab, zero), (tab, zero))
+        cache.update(0, blk(start), blk(start), start)
+        again = cache.block_key(start, 20, target)      # the in-place re-run of the same block (next step)
+        assert not again.appends and not again.rebase and again.evicted == 0
+    torch.cuda.synchronize()
+    assert keys[0].local_end == 0
+    assert keys[1].appends and keys[1].evicted == 0 and not keys[1].rebase
+    assert keys[3].rebase and keys[3].take_raw and keys[3].evicted == 20
+    assert keys[4].rebase and not keys[4].take_raw
+    assert keys[4] == keys[5]
+    p = [cache.pointers4(0)]
+    cache.set_pointers(p)
+    assert [cache.pointers4(0)] == p
+    # a block the cache cannot take is refused with the plan's message
+    with pytest.raises(fv.TensorError):
+        cache.block_key(1000, 20, 0)
