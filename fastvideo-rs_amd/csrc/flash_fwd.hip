@@ -50,8 +50,9 @@
 // instructions and no branches (a branch inside the unrolled phase breaks the
 // register allocation of the 16-register accumulator tuples: 59 spills measured).
 // Every wave waits for its own loads at the end of the same phase, one barrier
-// before phase m+1 of either group reads them. V buffers 2 and 3 start as zeros
-// (phase 0 multiplies them with P = 0). An odd tile count is rounded up: the extra
+// before phase m+1 of either group reads them. A dense walk's phase 0 has no previous pair and runs
+// its QK half only (unrolled apart from the loop); a masked walk keeps one loop, whose phase 0
+// multiplies V buffers 2 and 3, zero-filled at the start, with P = 0. An odd tile count is rounded up: the extra
 // tile re-reads the last one and all its scores are masked. Tile indices are walk
 // positions: a masked call walks up to three ascending tile ranges (block-causal:
 // sink tiles, then the band; VDN window: rows before the video + frame 0, the
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             Dma::issue_prepared(a1, it);
         }
     }
-    {   // zero V buffers 2 and 3 (two tiles), an equal share per thread
+    if constexpr (MASKED) {   // zero V buffers 2 and 3 (two tiles), an equal share per thread
         const u32x4 z = {0u, 0u, 0u, 0u};
         constexpr int kPer = 2 * kTileBytes / 512;
         lds_u8* zb = smem + (kRing2 + 2) * kTileBytes + tid * kPer;
@@ -284,14 +285,23 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         }
     };
 
+    // A dense walk's first phase has no previous pair to multiply: it is unrolled apart (part 0) and
+    // runs the K groups only. Masked walks keep one loop (part 1 alone).
+#pragma unroll
+    for (int part = 0; part < 2; part++) {
+    const bool first = !MASKED && part == 0;
+    const int m_begin = (MASKED || part == 0) ? 0 : 1;
+    const int m_end = part == 0 ? (MASKED ? 0 : 1) : np;
 #pragma unroll 1
-    for (int m = 0; m < np; m++) {
+    for (int m = m_begin; m < m_end; m++) {
         // ---- matrix phase: group 0 in slot 2m, group 1 in slot 2m+1 ----
         __builtin_amdgcn_s_setprio(1);
         constexpr int kAhead = MASKED ? 2 : 3;
+        const int g0 = first ? D / 16 : 0;   // the first phase starts at the K groups
         // DMA issue slots: after groups 1, 2 (first tile of the pair) and 4, 5 (second) at
         // D = 128; after groups 1 and 3 at D = 64 (one instruction per tile and wave)
         auto hook_k = [&](int g) {
+            g -= g0;
             if constexpr (kIt == 2) {
                 if (g == 1) Dma::issue_prepared(dk0, 0);
                 if (g == 2) Dma::issue_prepared(dk0, 1);
@@ -303,6 +313,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             }
         };
         auto hook_v = [&](int g) {
+            g -= g0;
             if constexpr (kIt == 2) {
                 if (g == 1) Dma::issue_prepared(dv0, 0);
                 if (g == 2) Dma::issue_prepared(dv0, 1);
@@ -313,8 +324,13 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                 if (g == 3) Dma::issue_prepared(dv1, 0);
             }
         };
-        mfma_phase<true, kAhead, decltype(hook_k)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_k);
-        mfma_phase<true, kAhead, decltype(hook_v)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_v);
+        if (first) {
+            mfma_phase<false, kAhead, decltype(hook_k)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_k);
+            mfma_phase<false, kAhead, decltype(hook_v)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_v);
+        } else {
+            mfma_phase<true, kAhead, decltype(hook_k)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_k);
+            mfma_phase<true, kAhead, decltype(hook_v)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_v);
+        }
         __builtin_amdgcn_s_setprio(0);
         wait_vmcnt<0>();             // this wave's loads of this phase have landed
         __builtin_amdgcn_sched_barrier(0);
@@ -337,6 +353,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             block_barrier();
             __builtin_amdgcn_sched_barrier(0);
         }
+    }
     }
     // O += P V of the last pair (their V landed before the last barrier both groups passed)
     pv_tile<D>(vbuf(2 * np - 2), rb.v, pb0, o);
