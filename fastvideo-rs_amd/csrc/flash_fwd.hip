@@ -50,9 +50,8 @@
 // instructions and no branches (a branch inside the unrolled phase breaks the
 // register allocation of the 16-register accumulator tuples: 59 spills measured).
 // Every wave waits for its own loads at the end of the same phase, one barrier
-// before phase m+1 of either group reads them. A dense walk's phase 0 has no previous pair and runs
-// its QK half only (unrolled apart from the loop); a masked walk keeps one loop, whose phase 0
-// multiplies V buffers 2 and 3, zero-filled at the start, with P = 0. An odd tile count is rounded up: the extra
+// before phase m+1 of either group reads them. Phase 0 has no previous pair and runs its QK half only
+// (unrolled apart from the loop). An odd tile count is rounded up: the extra
 // tile re-reads the last one and all its scores are masked. Tile indices are walk
 // positions: a masked call walks up to three ascending tile ranges (block-causal:
 // sink tiles, then the band; VDN window: rows before the video + frame 0, the
@@ -216,19 +215,11 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             Dma::issue_prepared(a1, it);
         }
     }
-    if constexpr (MASKED) {   // zero V buffers 2 and 3 (two tiles), an equal share per thread
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        constexpr int kPer = 2 * kTileBytes / 512;
-        lds_u8* zb = smem + (kRing2 + 2) * kTileBytes + tid * kPer;
-#pragma unroll
-        for (int i = 0; i < kPer / 16; i++) lds_write_b128(zb + 16 * i, z);
-    }
     bf16x8 qf[D / 16];
     {
         const int row = wave * 32 + c32;
         load_q_frags<D>(Qh, row, row < qlen, lane, qf);   // drains vmcnt: K(0), K(1) have landed too
     }
-    __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the zero fill is in LDS
     const TileReadBases rb = tile_read_bases<D>(lane);
 
     constexpr int kNO = D / 32;   // 32-wide d blocks of the accumulator
@@ -240,7 +231,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     SoftmaxState st;
     st.init();
     f32x16 s0[2], s1[2];
-    bf16x8 pb0[4], pb1[4];     // P of the previous pair of tiles; zero before the first
+    bf16x8 pb0[4], pb1[4];     // P of the previous pair of tiles (first read in phase 1; defined from the start)
 #pragma unroll
     for (int t = 0; t < 4; t++)
 #pragma unroll
@@ -251,7 +242,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
 
     typename Dma::Prepared dk0 = target_k(2), dk1 = target_k(3), dv0 = target_v(0), dv1 = target_v(1);
 
-    block_barrier();                 // K(0), K(1), zeros resident
+    block_barrier();                 // K(0), K(1) resident
     if (grp == 1) block_barrier();   // group 1 idles through slot 0
 
     // scores of walk position e: keys past the end (or a position past the walk) to -inf;
@@ -285,13 +276,13 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         }
     };
 
-    // A dense walk's first phase has no previous pair to multiply: it is unrolled apart (part 0) and
-    // runs the K groups only. Masked walks keep one loop (part 1 alone).
+    // The first phase of a walk has no previous pair to multiply: it is unrolled apart (part 0) and runs
+    // the K groups only.
 #pragma unroll
     for (int part = 0; part < 2; part++) {
-    const bool first = !MASKED && part == 0;
-    const int m_begin = (MASKED || part == 0) ? 0 : 1;
-    const int m_end = part == 0 ? (MASKED ? 0 : 1) : np;
+    const bool first = part == 0;
+    const int m_begin = part == 0 ? 0 : 1;
+    const int m_end = part == 0 ? 1 : np;
 #pragma unroll 1
     for (int m = m_begin; m < m_end; m++) {
         // ---- matrix phase: group 0 in slot 2m, group 1 in slot 2m+1 ----
