@@ -373,7 +373,35 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             return;
         }
     }
-    if (row < qlen) {
+    if (out_is_bf16) {
+        // bf16 rows through this wave's own 32 x 2D-byte slice of the K ring (every K read is behind the last
+        // barrier and no load is in flight): scattered 8-byte pieces in, whole rows out, 16 bytes per
+        // lane and 1 KB (D = 128) of consecutive output per store instruction
+        constexpr int kRowB = 2 * kD, kCh = kRowB / 16;
+        lds_u8* my = smem + wave * (32 * kRowB);
+#pragma unroll
+        for (int db = 0; db < kNO; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                f32x4 r;
+#pragma unroll
+                for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
+                const bf16x4 rb4 = __builtin_convertvector(r, bf16x4);
+                const int ch = (4 * db + g) ^ (c32 & (kCh - 1));
+                *reinterpret_cast<__attribute__((address_space(3))) bf16x4*>(my + c32 * kRowB + (ch << 4) + 8 * h) = rb4;
+            }
+        // (same-wave LDS writes and reads complete in order; the compiler waits on the reads' data)
+        constexpr int kRowsPer = 64 / kCh;           // rows one store instruction covers
+        const int lr = lane / kCh, lc = lane % kCh;
+        uint16_t* ob = out_bf16 + ((size_t)bh * sq + q0 + wave * 32) * kD;
+#pragma unroll
+        for (int i = 0; i < 32 / kRowsPer; i++) {
+            const int rr = i * kRowsPer + lr;
+            const u32x4 val = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(
+                my + rr * kRowB + ((lc ^ (rr & (kCh - 1))) << 4));
+            if (wave * 32 + rr < qlen) *reinterpret_cast<u32x4*>(ob + (size_t)rr * kD + lc * 8) = val;
+        }
+    } else if (row < qlen) {
         const size_t base = ((size_t)bh * sq + q0 + row) * kD;
 #pragma unroll
         for (int db = 0; db < kNO; db++)
