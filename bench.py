@@ -138,7 +138,9 @@ def bench_kvcache(args, fpb=3):
     layer: 21/fpb cache writes + dense calls of Sq = fpb*1560 against Sk = Sq ... 32760, with the keys
     split over several workgroups where the query tiles alone do not fill the GPU (the library's own
     choice, fv_sdpa_splitkv_choose). The same with a contiguous copy of every window first (what the
-    reference's `narrow` does) and without split-KV is timed beside it."""
+    reference's `narrow` does) and without split-KV is timed beside it. A rollout is 40 to 90 short
+    launches, so each form is captured once as a HIP graph and the replays are timed (what a serving loop
+    does); the eager Python loop, whose time depends on the host, is reported beside it."""
     import torch
 
     import fv_sdpa
@@ -153,7 +155,6 @@ def bench_kvcache(args, fpb=3):
                   for _ in range(3))
     cache = fv_sdpa.CausalKvCache(fv_sdpa.KvSpec.global_window(ft, frames), 1)
     plan = fv_sdpa.Plan.kv_window()
-    stream = torch.cuda.current_stream().cuda_stream
     outs = [torch.empty((h, n, d), device=dev, dtype=torch.bfloat16) for _ in range(blocks)]
     scale = 1.0 / d ** 0.5
 
@@ -162,6 +163,7 @@ def bench_kvcache(args, fpb=3):
     splits_used = []
 
     def rollout(copy_windows, split=True):
+        stream = torch.cuda.current_stream().cuda_stream    # the capturing stream inside a graph capture
         cache.reset()
         for i in range(blocks):
             kw, vw = cache.update(0, ks[i], vs[i], i * n)
@@ -187,9 +189,18 @@ def bench_kvcache(args, fpb=3):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / args.steps
 
-    in_place = timed(lambda: rollout(False))
-    copied = timed(lambda: rollout(True, split=False))
-    unsplit = timed(lambda: rollout(False, split=False))
+    def timed_graph(fn):
+        fn()                                   # the layer's buffers exist before the capture
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        return timed(graph.replay)
+
+    eager = timed(lambda: rollout(False))
+    in_place = timed_graph(lambda: rollout(False))
+    copied = timed_graph(lambda: rollout(True, split=False))
+    unsplit = timed_graph(lambda: rollout(False, split=False))
     # the plan entry once, to show it takes the same route
     kw, vw = cache.update(0, ks[0], vs[0], 0)
     before = fv_sdpa.rt_stats()
@@ -206,6 +217,7 @@ def bench_kvcache(args, fpb=3):
                                "cache write + attention per block", "flops_per_step": flops,
                    "key_splits_per_block": splits_used},
         "ms_per_step_with_window_copies_no_split": round(copied, 4), "ms_per_step_in_place_no_split": round(unsplit, 4),
+        "ms_per_step_eager_python_loop": round(eager, 4),
         "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::flash_fwd_pp2<false, 128>"},
     }

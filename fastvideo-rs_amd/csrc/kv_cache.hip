@@ -22,6 +22,21 @@ __global__ __launch_bounds__(256) void kv_copy_rows_kernel(u32x4* __restrict__ d
     }
 }
 
+// The same copy for a K and a V tensor in one launch (blockIdx.y picks the tensor): a cache write or a
+// roll chunk moves both, and at these sizes a launch costs about what its copy does.
+struct KvCopyArgs {
+    u32x4* dst;
+    const u32x4* src;
+    size_t units, dst_plane, src_plane, dst_off, src_off, total;
+};
+__global__ __launch_bounds__(256) void kv_copy_rows_pair_kernel(KvCopyArgs a, KvCopyArgs b) {
+    const KvCopyArgs& c = blockIdx.y == 0 ? a : b;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < c.total; i += (size_t)gridDim.x * 256) {
+        const size_t r = i / c.units, u = i - r * c.units;
+        c.dst[r * c.dst_plane + c.dst_off + u] = c.src[r * c.src_plane + c.src_off + u];
+    }
+}
+
 // Interleaved RoPE on BHSD rows (kernels/core.cu:1933-1955 `apply_rotary_bshd` through
 // wan/causal.rs:250-262 `rope_bhsd_f32`): pair (2i, 2i+1) of row r turns by the angle whose cos / sin
 // sit in the EVEN slot 2i of the [s, d] tables; f32 arithmetic, products unfused, as the reference.
@@ -130,6 +145,52 @@ int kv_copy_tokens(void* dst, size_t dst_rows, size_t dst_off, const void* src, 
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? FV_OK : fv_fail_hip(e, "kv_copy_rows");
 }
+
+namespace {
+// Arguments of one tensor's copy, checked as kv_copy_tokens checks them. 0 = nothing to move.
+int kv_copy_args(void* dst, size_t dst_rows, size_t dst_off, const void* src, size_t src_rows, size_t src_off,
+                 size_t len, size_t bh, size_t d, DType dtype, fv::KvCopyArgs& out) {
+    out = fv::KvCopyArgs{nullptr, nullptr, 1, 0, 0, 0, 0, 0};
+    if (!dst || !src) return fv_invalid("kv copy: null operand");
+    if (dst_off + len > dst_rows || src_off + len > src_rows) return fv_invalid("kv copy: rows outside the buffers");
+    if (len == 0 || bh == 0) return FV_OK;
+    const size_t row_bytes = d * esize(dtype);
+    if (row_bytes == 0 || row_bytes % 16 != 0 || (((uintptr_t)dst | (uintptr_t)src) & 15) != 0)
+        return fv_decline("kv copy: rows must be 16-byte multiples at 16-byte aligned addresses");
+    const size_t ru = row_bytes / 16, units = len * ru;
+    if (bh > (size_t)LONG_MAX / (units ? units : 1)) return fv_decline("kv copy: too large");
+    out = fv::KvCopyArgs{(fv::u32x4*)dst, (const fv::u32x4*)src, units, dst_rows * ru, src_rows * ru, dst_off * ru,
+                         src_off * ru, units * bh};
+    return FV_OK;
+}
+
+// K and V of one cache write (or one roll chunk) in a single launch.
+int kv_copy_tokens_pair(const fv::KvCopyArgs& a, const fv::KvCopyArgs& b, hipStream_t st) {
+    const size_t most = std::max(a.total, b.total);
+    if (most == 0) return FV_OK;
+    const size_t blocks = std::min<size_t>((most + 255) / 256, 1u << 20);
+    hipLaunchKernelGGL(fv::kv_copy_rows_pair_kernel, dim3((unsigned)blocks, 2), dim3(256), 0, st, a, b);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FV_OK : fv_fail_hip(e, "kv_copy_rows_pair");
+}
+
+// The roll of K and V together: chunks no longer than the shift, so that no launch reads what it writes.
+int kv_shift_pair_down(void* k, void* v, size_t rows, size_t from, size_t to, size_t len, size_t bh, size_t d, size_t dv,
+                       DType kd, DType vd, hipStream_t st) {
+    if (to >= from) return len == 0 || to == from ? FV_OK : fv_invalid("kv shift: tokens only move down");
+    const size_t shift = from - to;
+    for (size_t done = 0; done < len;) {
+        const size_t n = std::min(shift, len - done);
+        fv::KvCopyArgs a, b;
+        int rc = kv_copy_args(k, rows, to + done, k, rows, from + done, n, bh, d, kd, a);
+        if (rc == FV_OK) rc = kv_copy_args(v, rows, to + done, v, rows, from + done, n, bh, dv, vd, b);
+        if (rc == FV_OK) rc = kv_copy_tokens_pair(a, b, st);
+        if (rc != FV_OK) return rc;
+        done += n;
+    }
+    return FV_OK;
+}
+}  // namespace
 
 int kv_shift_tokens_down(void* t, size_t rows, size_t from, size_t to, size_t len, size_t bh, size_t d, DType dtype,
                          hipStream_t st) {
@@ -294,8 +355,7 @@ Result<std::pair<Tensor, Tensor>> CausalKvCache::update(size_t layer, const Tens
         const size_t sink = std::min(spec.sink, prev);
         const size_t tail_start = std::min(sink + mv.evicted, prev), tail = prev - tail_start;
         if (tail > 0) {
-            int rc = kv_shift_tokens_down(L.k, L.cap, tail_start, sink, tail, bh, d, L.kd, st);
-            if (rc == FV_OK) rc = kv_shift_tokens_down(L.v, L.cap, tail_start, sink, tail, bh, dv, L.vd, st);
+            const int rc = kv_shift_pair_down(L.k, L.v, L.cap, tail_start, sink, tail, bh, d, dv, L.kd, L.vd, st);
             if (rc != FV_OK) return kv_msg(std::string("causal kv: roll: ") + fv_sdpa_last_error());
         }
         valid = sink + tail;
@@ -303,8 +363,10 @@ Result<std::pair<Tensor, Tensor>> CausalKvCache::update(size_t layer, const Tens
     if (mv.local_start + skip > valid)
         return kv_msg("causal kv: write at " + std::to_string(mv.local_start + skip) + " leaves a gap after " +
                       std::to_string(valid) + " cached tokens");
-    int rc = kv_copy_tokens(L.k, L.cap, mv.local_start + skip, k.data, n, skip, n - skip, bh, d, L.kd, st);
-    if (rc == FV_OK) rc = kv_copy_tokens(L.v, L.cap, mv.local_start + skip, v.data, n, skip, n - skip, bh, dv, L.vd, st);
+    fv::KvCopyArgs ca, cb;
+    int rc = kv_copy_args(L.k, L.cap, mv.local_start + skip, k.data, n, skip, n - skip, bh, d, L.kd, ca);
+    if (rc == FV_OK) rc = kv_copy_args(L.v, L.cap, mv.local_start + skip, v.data, n, skip, n - skip, bh, dv, L.vd, cb);
+    if (rc == FV_OK) rc = kv_copy_tokens_pair(ca, cb, st);
     if (rc != FV_OK) return kv_msg(std::string("causal kv: write: ") + fv_sdpa_last_error());
     L.global_end = current_start + n;
     L.local_end = mv.local_end;
