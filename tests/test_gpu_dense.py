@@ -190,6 +190,9 @@ def test_headline_shape_sampled_rows(fv, oracle):
     torch.cuda.synchronize()
     wantc = oracle.sdpa_composed_rows(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), rows)
     assert_parity(outc[:, torch.from_numpy(rows).cuda()].cpu().numpy(), wantc, "cross_headline_rows")
+    # the bf16 output (whole rows staged through LDS) is the RNE rounding of the f32 output, every element
+    assert torch.equal(fv.sdpa_dense_bf16(q, k, v, out_bf16=True), out.to(torch.bfloat16))
+    assert torch.equal(fv.sdpa_dense_bf16(q, kc, vc, out_bf16=True), outc.to(torch.bfloat16))
 
 
 def test_wan14b_shape_sampled_rows(fv, oracle):
