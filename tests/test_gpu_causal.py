@@ -117,6 +117,8 @@ def test_headline_causal_shape_sampled_rows(fv, oracle, bt):
     want = oracle.sdpa_composed_rows(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), rows,
                                      mask_bc=(bt, 0, 0))
     assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, f"causal_headline_{bt}")
+    # the bf16 output is the RNE rounding of the f32 output, every element
+    assert torch.equal(fv.sdpa_block_causal_bf16(q, k, v, bt, 0, 0, out_bf16=True), out.to(torch.bfloat16))
 
 
 @pytest.mark.parametrize("mode", ["block_causal", "vdn_window"])
