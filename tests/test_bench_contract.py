@@ -54,3 +54,15 @@ def test_headline_line_has_every_field_the_driver_reads():
     assert abs(rec["value"] - roof["achieved"]) / roof["achieved"] < 0.1
     cpu = rec["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["unit"] == "TFLOP/s" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("workload", ["tiny", "cross", "softmax", "machine", "kvcache1"])
+def test_other_workloads_emit_one_json_line(workload):
+    r = run(["--workload", workload, "--steps", "2", "--warmup", "1", "--cpu-seconds", "0"])
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [x for x in r.stdout.splitlines() if x.strip()]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    assert rec["n_gpus"] == 1 and rec["value"] > 0 and "workload" in rec["config"] and "roofline" in rec
+    assert rec["roofline"]["bound"] in ("mfma", "hbm") and 0 < rec["roofline"]["frac"] < 1.0
