@@ -25,3 +25,20 @@ def test_header_compiles_as_c_and_links(tmp_path):
     assert "shards=0,6,6,5 " in line                 # rt/sp.rs:66-74
     assert "backend=1 route=2:1,2 " in line
     assert "local_attn_size=-1 keeps a 21-frame KV window" in line   # the refused plan's message
+
+
+def test_oracle_c_functions_are_clean_under_address_and_undefined_sanitizers(tmp_path):
+    """The checker itself is checked: every C function of the oracle runs on odd small shapes in a
+    native build with -fsanitize=address,undefined (leak check on); any report aborts the driver."""
+    exe = str(tmp_path / "oracle_sanitize")
+    build = subprocess.run(["gcc", "-O1", "-g", "-std=c11", "-fopenmp", "-ffp-contract=off", "-fsanitize=address,undefined",
+                            "-fno-sanitize-recover=all", "-I", os.path.join(ROOT, "oracle"),
+                            os.path.join(ROOT, "tests", "c_abi", "oracle_sanitize.c"), os.path.join(ROOT, "oracle", "fv_oracle.c"),
+                            "-o", exe, "-lm"], capture_output=True, text=True)
+    if build.returncode != 0 and ("asan" in build.stderr.lower() or "sanitize" in build.stderr.lower()):
+        pytest.skip("this gcc has no sanitizer runtimes")
+    assert build.returncode == 0, build.stderr[-2000:]
+    env = dict(os.environ)
+    env["ASAN_OPTIONS"] = "detect_leaks=1:verify_asan_link_order=0"
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=120, env=env)
+    assert out.returncode == 0 and "oracle sanitizer run: ok" in out.stdout, (out.returncode, out.stdout[-500:], out.stderr[-3000:])
