@@ -15,10 +15,9 @@ constexpr int kTileElems = 64;   // VSA cube = 4x4x4 tokens (rt/vsa.rs:29-31)
 // same order and operations as the reference, so the result is bit-identical
 // to its host restatement.
 template <bool IN_BF16>
-__global__ __launch_bounds__(256) void vsa_tile_mean_kernel(
-    const void* __restrict__ x, const int* __restrict__ slot_src,
-    const int* __restrict__ block_sizes, float* __restrict__ out, long seq, int dim,
-    int num_tiles, int round16) {
+FV_DEV void tile_mean_body(const void* __restrict__ x, const int* __restrict__ slot_src,
+                           const int* __restrict__ block_sizes, float* __restrict__ out, long seq, int dim,
+                           int num_tiles, int round16) {
     const int grp = threadIdx.x >> 5, ln = threadIdx.x & 31;
     const int tile = blockIdx.x * 8 + grp;
     const long bh = blockIdx.y;
@@ -69,6 +68,26 @@ __global__ __launch_bounds__(256) void vsa_tile_mean_kernel(
         for (int e = 0; e < 4; e++) r[e] = n > 0 ? __fdiv_rn(acc[e], (float)n) : 0.0f;
         *reinterpret_cast<f32x4*>(ob + d0) = r;
     }
+}
+
+template <bool IN_BF16>
+__global__ __launch_bounds__(256) void vsa_tile_mean_kernel(
+    const void* __restrict__ x, const int* __restrict__ slot_src,
+    const int* __restrict__ block_sizes, float* __restrict__ out, long seq, int dim,
+    int num_tiles, int round16) {
+    tile_mean_body<IN_BF16>(x, slot_src, block_sizes, out, seq, dim, num_tiles, round16);
+}
+// q, k and v of the whole op in one launch (blockIdx.z picks the tensor)
+struct Three {
+    const void* in[3];
+    void* out[3];
+};
+template <bool IN_BF16>
+__global__ __launch_bounds__(256) void vsa_tile_mean3_kernel(Three t, const int* __restrict__ slot_src,
+                                                             const int* __restrict__ block_sizes, long seq, int dim,
+                                                             int num_tiles, int round16) {
+    tile_mean_body<IN_BF16>(t.in[blockIdx.z], slot_src, block_sizes, (float*)t.out[blockIdx.z], seq, dim, num_tiles,
+                            round16);
 }
 
 // ---- coarse scores (rt/vsa.rs:385-388) ---------------------------------------------
@@ -319,10 +338,8 @@ __global__ __launch_bounds__(256) void vsa_topk_kernel(const float* __restrict__
 // ---- tile permute (kernels/core.cu:1659-1672, kernels/attn3.cu:230-244) --------------
 // [bh, seq, 128] -> tile-contiguous bf16 [bh, padded, 128]; padding slots are zero.
 template <bool IN_BF16>
-__global__ __launch_bounds__(256) void vsa_tile_qkv_kernel(const void* __restrict__ x,
-                                                           const int* __restrict__ slot_src,
-                                                           uint16_t* __restrict__ xt, long seq,
-                                                           long padded, int dim) {
+FV_DEV void tile_qkv_body(const void* __restrict__ x, const int* __restrict__ slot_src, uint16_t* __restrict__ xt,
+                          long seq, long padded, int dim) {
     const long chunks = dim / 8;
     const long rem = blockIdx.x * 256L + threadIdx.x;
     if (rem >= padded * chunks) return;
@@ -345,6 +362,18 @@ __global__ __launch_bounds__(256) void vsa_tile_qkv_kernel(const void* __restric
         }
     }
     *reinterpret_cast<u32x4*>(xt + (bh * padded + slot) * dim + c * 8) = v;
+}
+template <bool IN_BF16>
+__global__ __launch_bounds__(256) void vsa_tile_qkv_kernel(const void* __restrict__ x,
+                                                           const int* __restrict__ slot_src,
+                                                           uint16_t* __restrict__ xt, long seq,
+                                                           long padded, int dim) {
+    tile_qkv_body<IN_BF16>(x, slot_src, xt, seq, padded, dim);
+}
+template <bool IN_BF16>
+__global__ __launch_bounds__(256) void vsa_tile_qkv3_kernel(Three t, const int* __restrict__ slot_src, long seq,
+                                                            long padded, int dim) {
+    tile_qkv_body<IN_BF16>(t.in[blockIdx.z], slot_src, (uint16_t*)t.out[blockIdx.z], seq, padded, dim);
 }
 
 // ---- fine stage (kernels/core.cu:1029-1179) ---------------------------------------------
@@ -555,6 +584,32 @@ extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16,
     else
         hipLaunchKernelGGL(vsa_tile_mean_kernel<false>, grid, block, 0, st, x, slot_src, block_sizes, out,
                            (long)seq, dim, num_tiles, round16);
+    return hipGetLastError();
+}
+
+// q, k and v in one launch each for the tile pass and the tile means (the whole op's order: the pass first,
+// the means from its bf16 output when mean_from_tiles, else from the operands where they lie).
+extern "C" hipError_t fv_internal_launch_tile_qkv3(const void* const x[3], int x_is_bf16, const int* slot_src,
+                                                   uint16_t* const xt[3], size_t bh, size_t seq, size_t padded, int dim,
+                                                   hipStream_t st) {
+    Three t;
+    for (int i = 0; i < 3; i++) t.in[i] = x[i], t.out[i] = xt[i];
+    const size_t per = padded * (size_t)(dim / 8);
+    const dim3 grid((unsigned)((per + 255) / 256), (unsigned)bh, 3), block(256);
+    if (x_is_bf16) hipLaunchKernelGGL(vsa_tile_qkv3_kernel<true>, grid, block, 0, st, t, slot_src, (long)seq, (long)padded, dim);
+    else hipLaunchKernelGGL(vsa_tile_qkv3_kernel<false>, grid, block, 0, st, t, slot_src, (long)seq, (long)padded, dim);
+    return hipGetLastError();
+}
+extern "C" hipError_t fv_internal_launch_tile_mean3(const void* const x[3], int x_is_bf16, const int* slot_src,
+                                                    const int* block_sizes, float* const out[3], size_t bh, size_t seq,
+                                                    int dim, int num_tiles, hipStream_t st) {
+    Three t;
+    for (int i = 0; i < 3; i++) t.in[i] = x[i], t.out[i] = out[i];
+    const dim3 grid((num_tiles + 7) / 8, (unsigned)bh, 3), block(256);
+    if (x_is_bf16)
+        hipLaunchKernelGGL(vsa_tile_mean3_kernel<true>, grid, block, 0, st, t, slot_src, block_sizes, (long)seq, dim, num_tiles, 0);
+    else
+        hipLaunchKernelGGL(vsa_tile_mean3_kernel<false>, grid, block, 0, st, t, slot_src, block_sizes, (long)seq, dim, num_tiles, 0);
     return hipGetLastError();
 }
 
