@@ -128,19 +128,17 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     int a_hi = 0, c_lo = 0x7fffffff, w_lo = 0, w_hi = 0;
     if constexpr (MASKED) {
         const int qi = q0 + wave * 32 + c32;   // this lane's query (rows past sq are never stored)
-        int b0, b1, b2 = 0;
+        const TileWalk w = mask_tile_walk(p, q0, qlen, nkt);
+        a1 = w.a1;
+        a2 = w.a2;
+        n0 = w.n0;
+        n1 = w.n1;
+        ne = w.ne;
         if (p.mask_mode == 1) {
             // block-causal (rt/attn.rs:449-453): keys of blocks (tq - win, tq], plus the sink blocks
             const int ft = p.ft, win = p.win;
-            const int fq_lo = q0 / ft, fq_hi = (q0 + qlen - 1) / ft;
-            const int hi_tok = (int)min((long)sk, (long)(fq_hi + 1) * ft);
-            const int lo_tok = min(hi_tok, win > 0 ? max(0, fq_lo - win + 1) * ft : 0);
-            const int sink_tok = (int)min((long)sk, (long)p.sink * ft);
-            b0 = (sink_tok + kBN - 1) / kBN;                       // sink tiles [0, b0)
-            a1 = lo_tok / kBN;                                     // band [a1, b1)
-            b1 = (hi_tok + kBN - 1) / kBN;
             const int tq = qi / ft;
-            a_hi = sink_tok;
+            a_hi = (int)min((long)sk, (long)p.sink * ft);
             w_hi = (int)min((long)0x7fffffff, (long)(tq + 1) * ft);
             w_lo = win > 0 ? max(0, tq - win + 1) * ft : 0;
         } else {
@@ -149,18 +147,6 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             const int vs = p.vs, ve = p.ve, t = p.ft, last = p.frames - 1, c = p.chunk, r = p.radius;
             auto lo_frame = [&](int f) { return max(0, c > 0 ? (f / c - r) * c : f - r); };
             auto hi_frame = [&](int f) { return min(last, c > 0 ? (f / c + r + 1) * c - 1 : f + r); };
-            const bool inner_tile = q0 >= vs + t && q0 + qlen <= ve - t;   // frames 1 .. last-1 only
-            if (inner_tile) {
-                const int fmin = (q0 - vs) / t, fmax = (q0 + qlen - 1 - vs) / t;
-                b0 = (vs + t + kBN - 1) / kBN;                     // rows before the video + frame 0
-                a1 = (vs + lo_frame(fmin) * t) / kBN;              // the window frames of the tile
-                b1 = (vs + (hi_frame(fmax) + 1) * t + kBN - 1) / kBN;
-                a2 = (ve - t) / kBN;                               // last frame + rows after the video
-                b2 = nkt;
-            } else {
-                b0 = nkt;
-                b1 = 0;
-            }
             const bool inner_q = qi >= vs + t && qi < ve - t;
             if (inner_q) {
                 const int qf = (qi - vs) / t;
@@ -172,17 +158,20 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                 a_hi = 0x7fffffff;
             }
         }
-        // ranges may touch or overlap: each starts no earlier than the previous one ends
-        b0 = min(b0, nkt);
-        a1 = max(a1, b0);
-        b1 = min(max(b1, a1), nkt);
-        a2 = max(a2, b1);
-        b2 = max(b2, a2);
-        n0 = b0;
-        n1 = b1 - a1;
-        ne = n0 + n1 + (min(b2, nkt) - min(a2, nkt));
     }
-    if (ne <= 0) return;   // cannot happen for sk >= 1 (a walk always holds the query's own keys)
+    if constexpr (MASKED) {
+        // No key tile is visible to any query of this tile (block-causal with more queries than keys
+        // and a window that has moved past the last key): rows of zeros, what a query without a
+        // visible key gets in a partly visible tile too (l == 0). Workgroup-uniform, before any barrier.
+        if (ne <= 0) {
+            const int units = kD * (out_is_bf16 ? 2 : 4) / 16;   // 16-byte units per output row
+            char* ob = out_is_bf16 ? (char*)(out_bf16 + ((size_t)bh * sq + q0) * kD)
+                                   : (char*)(out_f32 + ((size_t)bh * sq + q0) * kD);
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            for (int u = tid; u < qlen * units; u += 512) *reinterpret_cast<u32x4*>(ob + (size_t)u * 16) = zero;
+            return;
+        }
+    }
     const int np = (ne + 1) / 2;             // phases
     // first key of walk position e; positions past the end repeat the last tile (their scores are masked)
     auto kv0_of = [&](int e) -> int {

@@ -124,6 +124,30 @@ void fv_vdn_window_dense_mask(size_t video_start, size_t frame_tokens, size_t fr
                 fv_vdn_window_allows(video_start, frame_tokens, frames, chunk, radius, q, k) ? 0.0f : -1e9f;
 }
 
+int fv_block_causal_tile_walk(size_t block_tokens, size_t window, size_t sink, size_t sq, size_t sk, size_t q0,
+                              int out4[4]) {
+    const size_t lim = (size_t)INT_MAX;
+    const size_t bm = (size_t)fv_internal_flash_block_m();
+    if (!out4) return fv_invalid("block_causal_tile_walk: null output");
+    if (block_tokens == 0 || window > lim || sink > lim || sq == 0 || sk == 0 || q0 >= sq || q0 % bm != 0 ||
+        (sq > sk ? sq : sk) + block_tokens > lim)
+        return fv_decline("block_causal_tile_walk: parameters outside the kernel's range");
+    fv::FlashParams p{};
+    p.mask_mode = 1;
+    p.sq = (int)sq;
+    p.sk = (int)sk;
+    p.ft = (int)block_tokens;
+    p.win = (int)window;
+    p.sink = (int)sink;
+    const int qlen = (int)(sq - q0 < bm ? sq - q0 : bm);
+    const fv::TileWalk w = fv::mask_tile_walk(p, (int)q0, qlen, (int)((sk + 63) / 64));
+    out4[0] = w.n0;
+    out4[1] = w.a1;
+    out4[2] = w.n1;
+    out4[3] = w.ne;
+    return FV_OK;
+}
+
 int fv_block_causal_for(size_t num_frames_per_block, long long local_attn_size, size_t frame_tokens,
                         size_t out3[3]) {
     const size_t fpb = num_frames_per_block ? num_frames_per_block : 1;

@@ -55,6 +55,65 @@ struct VsaFineParams {
     long seq;
 };
 
+// The key-tile walk of one query tile of a masked launch: up to three ascending, non-overlapping
+// ranges of 64-key tiles, [0, n0), [a1, a1 + n1) and [a2, a2 + n2), ne = n0 + n1 + n2 tiles in all
+// (ne == 0: no query of the tile sees any key). Every key visible to any query of the tile lies in
+// a walked tile; which scores inside a walked tile count is decided per lane.
+//   block-causal (rt/attn.rs:449-453): the sink tiles, then the band of the tile's blocks;
+//   VDN window (rt/attn.rs:483-510): rows before the video + frame 0, the window frames of the
+//   tile, the last frame + rows after the video; a tile holding an anchor / global row walks all.
+struct TileWalk {
+    int a1, a2, n0, n1, ne;
+};
+__host__ __device__ inline TileWalk mask_tile_walk(const FlashParams& p, int q0, int qlen, int nkt) {
+    constexpr int kKeys = 64;
+    const int sk = p.sk;
+    auto imin = [](int a, int b) { return a < b ? a : b; };
+    auto imax = [](int a, int b) { return a > b ? a : b; };
+    int a1 = 0, a2 = 0, b0, b1, b2 = 0;
+    if (p.mask_mode == 1) {
+        const int ft = p.ft, win = p.win;
+        const int fq_lo = q0 / ft, fq_hi = (q0 + qlen - 1) / ft;
+        const long hi_l = (long)(fq_hi + 1) * ft;
+        const int hi_tok = (int)(hi_l < (long)sk ? hi_l : (long)sk);
+        const int lo_tok = imin(hi_tok, win > 0 ? imax(0, fq_lo - win + 1) * ft : 0);
+        const long sink_l = (long)p.sink * ft;
+        const int sink_tok = (int)(sink_l < (long)sk ? sink_l : (long)sk);
+        b0 = (sink_tok + kKeys - 1) / kKeys;
+        a1 = lo_tok / kKeys;
+        b1 = (hi_tok + kKeys - 1) / kKeys;
+    } else {
+        const int vs = p.vs, ve = p.ve, t = p.ft, last = p.frames - 1, c = p.chunk, r = p.radius;
+        auto lo_frame = [&](int f) { return imax(0, c > 0 ? (f / c - r) * c : f - r); };
+        auto hi_frame = [&](int f) { return imin(last, c > 0 ? (f / c + r + 1) * c - 1 : f + r); };
+        const bool inner_tile = q0 >= vs + t && q0 + qlen <= ve - t;   // frames 1 .. last-1 only
+        if (inner_tile) {
+            const int fmin = (q0 - vs) / t, fmax = (q0 + qlen - 1 - vs) / t;
+            b0 = (vs + t + kKeys - 1) / kKeys;
+            a1 = (vs + lo_frame(fmin) * t) / kKeys;
+            b1 = (vs + (hi_frame(fmax) + 1) * t + kKeys - 1) / kKeys;
+            a2 = (ve - t) / kKeys;
+            b2 = nkt;
+        } else {
+            b0 = nkt;
+            b1 = 0;
+        }
+    }
+    // ranges may touch or overlap: each starts no earlier than the previous one ends
+    b0 = imin(b0, nkt);
+    a1 = imax(a1, b0);
+    b1 = imin(imax(b1, a1), nkt);
+    a2 = imax(a2, b1);
+    b2 = imax(b2, a2);
+    TileWalk w;
+    w.a1 = a1;
+    w.a2 = a2;
+    w.n0 = b0;
+    w.n1 = b1 - a1;
+    w.ne = w.n0 + w.n1 + (imin(b2, nkt) - imin(a2, nkt));
+    return w;
+}
+
 }  // namespace fv
 
 extern "C" int fv_internal_flash_block_m(void);   // queries per workgroup of the flash kernel in use

@@ -1,5 +1,5 @@
 // Video Sparse Attention stages for gfx950: tile mean, coarse scores, coarse
-// softmax x V, radix-select top-k, tile permute, block-sparse fine attention,
+// softmax x V, bitwise-descent top-k, tile permute, block-sparse fine attention,
 // gated combine. Reference stages: crates/fastvideo-cudarc/src/rt/vsa.rs:358-470
 // and the kernels cited per function below (kernels/core.cu, kernels/attn3.cu).
 #include "attn_core.h"
@@ -90,53 +90,55 @@ __global__ __launch_bounds__(256) void vsa_tile_mean3_kernel(Three t, const int*
                             round16);
 }
 
-// ---- coarse scores (rt/vsa.rs:385-388) ---------------------------------------------
-// scores[bh, qt, kt] = (sum over d ascending of qc*kc, f32 mul then add) * scale.
-// The reference runs cuBLAS f32 here; a fixed summation order makes the scores,
-// and so the top-k selection, reproducible bit for bit on the host.
+// ---- coarse scores (rt/vsa.rs:385-388; arithmetic of the host oracle, rt/vsa.rs:185-189) ----
+// scores[bh, qt, kt] = f32( (f64 dot of the tile means, d ascending from -0.0) * f64(scale) ).
+// The product of two f32 values is exact in f64, so one v_fma_f64 per term is the oracle's
+// multiply-then-add, and the scores (and with them the selected tiles) equal the host oracle's
+// bit for bit. (The reference's device path runs cuBLAS f32 here, whose order is unspecified.)
+// A 64 x 64 block of scores per workgroup, 4 x 4 per thread, the means staged in LDS as f32.
 __global__ __launch_bounds__(256) void vsa_coarse_scores_kernel(
     const float* __restrict__ qc, const float* __restrict__ kc, float* __restrict__ scores,
     int nb, int dim, float scale) {
-#pragma clang fp contract(off)   // keep mul and add separate: the order is part of the contract
-    __shared__ float qs[64][33];
-    __shared__ float ks[64][33];
+    __shared__ float qs[32][65];   // [d][tile]: the 4 tiles of a thread are consecutive words
+    __shared__ float ks[32][65];
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int q0 = blockIdx.y * 64, k0 = blockIdx.x * 64;
     const long bh = blockIdx.z;
     const float* qb = qc + bh * nb * (long)dim;
     const float* kb = kc + bh * nb * (long)dim;
-    float acc[4][4];
+    double acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = 0.f;
+        for (int j = 0; j < 4; j++) acc[i][j] = -0.0;   // the identity of Rust's f64 Sum
     for (int d0 = 0; d0 < dim; d0 += 32) {
         for (int e = threadIdx.x; e < 64 * 32; e += 256) {
             const int r = e >> 5, c = e & 31;
-            qs[r][c] = (q0 + r < nb && d0 + c < dim) ? qb[(long)(q0 + r) * dim + d0 + c] : 0.f;
-            ks[r][c] = (k0 + r < nb && d0 + c < dim) ? kb[(long)(k0 + r) * dim + d0 + c] : 0.f;
+            qs[c][r] = (q0 + r < nb && d0 + c < dim) ? qb[(long)(q0 + r) * dim + d0 + c] : 0.f;
+            ks[c][r] = (k0 + r < nb && d0 + c < dim) ? kb[(long)(k0 + r) * dim + d0 + c] : 0.f;
         }
         __syncthreads();
         const int dn = min(32, dim - d0);
         for (int c = 0; c < dn; c++) {
-            float a[4], b[4];
+            double a[4], b[4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) a[i] = qs[ty * 4 + i][c];
+            for (int i = 0; i < 4; i++) a[i] = (double)qs[c][ty * 4 + i];
 #pragma unroll
-            for (int j = 0; j < 4; j++) b[j] = ks[tx * 4 + j][c];
+            for (int j = 0; j < 4; j++) b[j] = (double)ks[c][tx * 4 + j];
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = acc[i][j] + a[i] * b[j];
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_fma(a[i], b[j], acc[i][j]);
         }
         __syncthreads();
     }
+    const double sc = (double)scale;
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int qi = q0 + ty * 4 + i, kj = k0 + tx * 4 + j;
-            if (qi < nb && kj < nb) scores[(bh * nb + qi) * (long)nb + kj] = acc[i][j] * scale;
+            if (qi < nb && kj < nb) scores[(bh * nb + qi) * (long)nb + kj] = (float)(acc[i][j] * sc);
         }
 }
 
@@ -215,124 +217,70 @@ __global__ __launch_bounds__(256) void vsa_coarse_pv_kernel(
 }
 
 // ---- top-k (kernels/core.cu:576-619, kernels/attn3.cu:279-363) ----------------------
-// T = k-th largest sortable key of the row (8-bit radix select, 4 histogram
-// passes over the row held in LDS); output = indices with key > T ascending,
-// then key == T ascending, up to k, zero padded. Bit-exact integer work.
+// Output contract: T = the k-th largest sortable key of the row; the indices whose key is
+// above T in ascending order, then those equal to T in ascending order, k in all, zero padded
+// (k > n: every index, then zeros). Integer work, bit-exact.
+//
+// One wave owns one row and keeps it in registers: lane l holds the keys of indices
+// l, 64 + l, 128 + l, ... (KPL of them; slots past n hold key 0 and are never emitted).
+// T is built bit by bit from the top: a bit stays set if at least k keys are >= the candidate.
+// A count is the sum of the popcounts of KPL wave-wide compare masks, so it lands in a scalar
+// register and the decision is a scalar branch: no LDS, no atomics, no barrier. The emit pass
+// walks the registers in index order; a lane's output slot is the running total plus the number
+// of set mask bits below it.
 FV_DEV unsigned sortable_key(float x) {
     const unsigned u = __builtin_bit_cast(unsigned, x);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
 constexpr int kTopkMaxN = 4096;
+constexpr int kTopkRowsPerBlock = 4;
 
-__global__ __launch_bounds__(256) void vsa_topk_kernel(const float* __restrict__ scores,
-                                                       unsigned* __restrict__ out, int rows,
-                                                       int n, int k) {
-    __shared__ unsigned keys[kTopkMaxN];
-    __shared__ unsigned hist[256];
-    __shared__ unsigned sel_prefix, sel_rem;
-    __shared__ unsigned wsum_gt[4], wsum_eq[4];
-    const int row = blockIdx.x;
-    if (row >= rows) return;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+FV_DEV int lanes_below(unsigned long long m) {
+    return (int)__builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
+}
+
+template <int KPL>
+__global__ __launch_bounds__(64 * kTopkRowsPerBlock) void vsa_topk_kernel(const float* __restrict__ scores,
+                                                                          unsigned* __restrict__ out, int rows,
+                                                                          int n, int k) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * kTopkRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= rows) return;   // the whole wave leaves; waves never meet at a barrier
     const float* s = scores + (long)row * n;
-    for (int i = tid; i < n; i += 256) keys[i] = sortable_key(s[i]);
-    if (tid == 0) {
-        sel_prefix = 0u;
-        sel_rem = (unsigned)k;
+    unsigned key[KPL];
+#pragma unroll
+    for (int j = 0; j < KPL; j++) {
+        const int i = 64 * j + lane;
+        key[j] = i < n ? sortable_key(s[i]) : 0u;
     }
-    __syncthreads();
-    unsigned thr = 0u;
+    unsigned t = 0u;           // k > n: threshold 0 lets every index through
     if (k <= n) {
 #pragma unroll 1
-        for (int pass = 0; pass < 4; pass++) {
-            const int shift = 24 - 8 * pass;
-            const unsigned hi_mask = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8));
-            hist[tid] = 0u;
-            __syncthreads();
-            const unsigned prefix = sel_prefix;
-            for (int i = tid; i < n; i += 256) {
-                const unsigned key = keys[i];
-                if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
-            }
-            __syncthreads();
-            if (wave == 0) {
-                // lane l owns bins [4l, 4l+4); suffix counts from the top bin down
-                unsigned c[4];
+        for (unsigned bit = 0x80000000u; bit != 0u; bit >>= 1) {
+            const unsigned cand = t | bit;
+            int at_least = 0;
 #pragma unroll
-                for (int b = 0; b < 4; b++) c[b] = hist[lane * 4 + b];
-                const unsigned local = c[0] + c[1] + c[2] + c[3];
-                unsigned suffix = local;
-#pragma unroll
-                for (int off = 1; off < 64; off <<= 1) {
-                    const unsigned o = __shfl_down(suffix, off);
-                    if (lane + off < 64) suffix += o;
-                }
-                const unsigned rem = sel_rem;
-                const unsigned above = suffix - local;
-                if (above < rem && suffix >= rem) {
-                    unsigned acc = above;
-                    int b = 3;
-                    for (; b > 0; b--) {
-                        if (acc + c[b] >= rem) break;
-                        acc += c[b];
-                    }
-                    sel_prefix = prefix | ((unsigned)(lane * 4 + b) << shift);
-                    sel_rem = rem - acc;
-                }
-            }
-            __syncthreads();
-        }
-        thr = sel_prefix;
-    }
-    // ordered compaction: thread t owns the contiguous index range [t*C, (t+1)*C)
-    const int C = (n + 255) / 256;
-    const int i0 = min(n, tid * C), i1 = min(n, i0 + C);
-    unsigned cgt = 0, ceq = 0;
-    for (int i = i0; i < i1; i++) {
-        const unsigned key = keys[i];
-        cgt += key > thr;
-        ceq += key == thr;
-    }
-    // exclusive scans over the block
-    unsigned sgt = cgt, seq_ = ceq;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const unsigned a = __shfl_up(sgt, off), b = __shfl_up(seq_, off);
-        if (lane >= off) {
-            sgt += a;
-            seq_ += b;
+            for (int j = 0; j < KPL; j++)
+                at_least += __builtin_popcountll(__builtin_amdgcn_ballot_w64(key[j] >= cand));
+            if (at_least >= k) t = cand;
         }
     }
-    if (lane == 63) {
-        wsum_gt[wave] = sgt;
-        wsum_eq[wave] = seq_;
-    }
-    __syncthreads();
-    unsigned base_gt = 0, base_eq = 0, tot_gt = 0, tot_eq = 0;
-#pragma unroll
-    for (int w = 0; w < 4; w++) {
-        if (w < wave) {
-            base_gt += wsum_gt[w];
-            base_eq += wsum_eq[w];
-        }
-        tot_gt += wsum_gt[w];
-        tot_eq += wsum_eq[w];
-    }
-    unsigned pgt = base_gt + sgt - cgt;
-    unsigned peq = tot_gt + base_eq + seq_ - ceq;
     unsigned* dst = out + (long)row * k;
-    for (int i = i0; i < i1; i++) {
-        const unsigned key = keys[i];
-        if (key > thr) {
-            if (pgt < (unsigned)k) dst[pgt] = (unsigned)i;
-            pgt++;
-        } else if (key == thr) {
-            if (peq < (unsigned)k) dst[peq] = (unsigned)i;
-            peq++;
+    int filled = 0;            // wave-uniform count of slots written so far
+#pragma unroll
+    for (int pass = 0; pass < 2; pass++) {
+#pragma unroll
+        for (int j = 0; j < KPL; j++) {
+            const int i = 64 * j + lane;
+            const bool take = i < n && (pass == 0 ? key[j] > t : key[j] == t);
+            const unsigned long long m = __builtin_amdgcn_ballot_w64(take);
+            const int pos = filled + lanes_below(m);
+            if (take && pos < k) dst[pos] = (unsigned)i;
+            filled += __builtin_popcountll(m);
         }
     }
-    for (unsigned pos = tot_gt + tot_eq + tid; pos < (unsigned)k; pos += 256) dst[pos] = 0u;
+    for (int pos = filled + lane; pos < k; pos += 64) dst[pos] = 0u;
 }
 
 // ---- tile permute (kernels/core.cu:1659-1672, kernels/attn3.cu:230-244) --------------
@@ -637,7 +585,14 @@ extern "C" hipError_t fv_internal_launch_coarse(const float* qc, const float* kc
 
 extern "C" hipError_t fv_internal_launch_topk(const float* scores, unsigned* out, int rows, int n, int k,
                                               hipStream_t st) {
-    hipLaunchKernelGGL(vsa_topk_kernel, dim3(rows), dim3(256), 0, st, scores, out, rows, n, k);
+    if (n < 1 || n > kTopkMaxN) return hipErrorInvalidValue;
+    const dim3 grid((rows + kTopkRowsPerBlock - 1) / kTopkRowsPerBlock), block(64 * kTopkRowsPerBlock);
+    // keys per lane: the smallest of 4, 8, 16, 32, 64 that holds the row
+    if (n <= 256) hipLaunchKernelGGL(vsa_topk_kernel<4>, grid, block, 0, st, scores, out, rows, n, k);
+    else if (n <= 512) hipLaunchKernelGGL(vsa_topk_kernel<8>, grid, block, 0, st, scores, out, rows, n, k);
+    else if (n <= 1024) hipLaunchKernelGGL(vsa_topk_kernel<16>, grid, block, 0, st, scores, out, rows, n, k);
+    else if (n <= 2048) hipLaunchKernelGGL(vsa_topk_kernel<32>, grid, block, 0, st, scores, out, rows, n, k);
+    else hipLaunchKernelGGL(vsa_topk_kernel<64>, grid, block, 0, st, scores, out, rows, n, k);
     return hipGetLastError();
 }
 

@@ -76,6 +76,7 @@ SIGNATURES = {
     "fv_block_causal_allows": (C.c_int, [_sz, _sz, _sz, _sz, _sz]),
     "fv_block_causal_dense_mask": (None, [_sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_block_causal_for": (C.c_int, [_sz, C.c_longlong, _sz, _vp]),
+    "fv_block_causal_tile_walk": (C.c_int, [_sz, _sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_sp_shard_ranges": (None, [_sz, _sz, _vp]),
     "fv_sdpa_vdn_window_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float,
                                           _sz, _sz, _sz, _sz, _sz, _vp]),

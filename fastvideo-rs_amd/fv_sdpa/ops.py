@@ -97,10 +97,14 @@ def sdpa_dense_bf16_splitkv(q, k, v, splits=None, scale=None, out_bf16=False):
     return out
 
 
-def sdpa_block_causal_bf16(q, k, v, block_tokens, window=0, sink=0, scale=None, out_bf16=False):
+def sdpa_block_causal_bf16(q, k, v, block_tokens, window=0, sink=0, scale=None, out_bf16=False, out=None):
     bh, sq, sk, d = _bhsd(q, k, v)
     scale = 1.0 / math.sqrt(d) if scale is None else scale
-    out = torch.empty((bh, sq, d), device=q.device, dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    want = torch.bfloat16 if out_bf16 else torch.float32
+    if out is None:
+        out = torch.empty((bh, sq, d), device=q.device, dtype=want)
+    elif out.dtype != want or tuple(out.shape) != (bh, sq, d) or not out.is_contiguous() or out.device != q.device:
+        raise ValueError(f"out must be a contiguous {want} tensor of shape {(bh, sq, d)} on {q.device}")
     _lib.check(_lib.lib().fv_sdpa_block_causal_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                                     int(out_bf16), bh, sq, sk, d, scale, block_tokens, window,
                                                     sink, _stream()))

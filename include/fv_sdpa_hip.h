@@ -375,6 +375,14 @@ void fv_vdn_window_dense_mask(size_t video_start, size_t frame_tokens, size_t fr
  * token window does not cover whole blocks. */
 int fv_block_causal_for(size_t num_frames_per_block, long long local_attn_size, size_t frame_tokens,
                         size_t out3[3]);
+/* The key tiles (64 keys each) that the fused block-causal kernel walks for the 256 queries starting at
+ * q0 (a multiple of 256): the loop bounds of the causal kernel body (kernels/attn2.cu:214-221), here up
+ * to two ascending tile ranges, out4 = {0 .. n0 (sink tiles), a1 .. a1 + n1 (the band)} as
+ * {n0, a1, n1, total}. total == 0: no query of the tile sees a key and its rows come out as zeros.
+ * Host arithmetic only (the kernel runs the same function); 0, or FV_DECLINED for parameters the
+ * kernel does not take. */
+int fv_block_causal_tile_walk(size_t block_tokens, size_t window, size_t sink, size_t sq, size_t sk, size_t q0,
+                              int out4[4]);
 /* rt/sp.rs:16-28 `shard_ranges`: out[world][2] = (start, len). The library itself never
  * shards (the full sequence stays on one GPU); kept for callers that do. */
 void fv_sp_shard_ranges(size_t seq, size_t world, size_t* out);

@@ -444,6 +444,9 @@ void fvo_vsa_combine(const float* sparse, const float* coarse, const float* gate
         }
 }
 
+/* C/rt/vsa.rs:185-189: the score of (query tile, key tile) is the f64 dot of the two tile means, d ascending,
+ * times f64(scale), cast to f32. The sum starts from -0.0, the identity of Rust's `Sum for f64` at the reference's
+ * pinned toolchain (>= 1.88): a dot whose every product is -0.0 stays -0.0, which total_cmp orders below +0.0. */
 void fvo_vsa_coarse_scores(const float* qc, const float* kc, float* scores, size_t bh, size_t nb,
                            size_t dim, float scale) {
     for (size_t b = 0; b < bh; b++)
@@ -451,9 +454,9 @@ void fvo_vsa_coarse_scores(const float* qc, const float* kc, float* scores, size
             for (size_t kt = 0; kt < nb; kt++) {
                 const float* a = qc + (b * nb + qt) * dim;
                 const float* c = kc + (b * nb + kt) * dim;
-                float acc = 0.0f;
-                for (size_t d = 0; d < dim; d++) acc += a[d] * c[d];
-                scores[(b * nb + qt) * nb + kt] = acc * scale;
+                double dot = -0.0;
+                for (size_t d = 0; d < dim; d++) dot += (double)a[d] * (double)c[d];
+                scores[(b * nb + qt) * nb + kt] = (float)(dot * (double)scale);
             }
 }
 
@@ -504,7 +507,7 @@ int fvo_vsa_attention_host(const float* q, const float* k, const float* v, const
         for (size_t qt = 0; qt < nb; qt++) {
             float* s = scores + qt * nb;
             for (size_t kt = 0; kt < nb; kt++) {
-                double dot = 0.0;
+                double dot = -0.0;   /* the identity of Rust's f64 Sum */
                 for (size_t d = 0; d < dim; d++)
                     dot += (double)qc[qt * dim + d] * (double)kc[kt * dim + d];
                 s[kt] = (float)(dot * (double)scale);
@@ -538,7 +541,7 @@ int fvo_vsa_attention_host(const float* q, const float* k, const float* v, const
                     const size_t kt = picks[pi];
                     for (size_t kslot = kt * TE; kslot < kt * TE + block_sizes[kt]; kslot++) {
                         const size_t ktok = (size_t)slot_src[kslot];
-                        double dot = 0.0;
+                        double dot = -0.0;
                         for (size_t d = 0; d < dim; d++)
                             dot += (double)qr[d] * (double)k[base + ktok * dim + d];
                         const float s = (float)(dot * (double)scale);

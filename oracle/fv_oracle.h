@@ -132,9 +132,10 @@ void fvo_vsa_tile_mean(const float* x, const int32_t* slot_src, const uint32_t* 
 void fvo_vsa_combine(const float* sparse, const float* coarse, const float* gate, const int32_t* slot_src,
                      float* out, size_t bh, size_t seq, size_t dim, size_t nb, size_t q_base,
                      size_t q_tiles, int round16);
-/* C/rt/vsa.rs:385-394 restated with a fixed accumulation order (the reference
- * uses cuBLAS f32, whose order is unspecified): scores[qt,kt] =
- * (sum_d in ascending d of qc*kc, f32, no FMA) * scale. */
+/* C/rt/vsa.rs:185-189 (stage 2 of vsa_attention_host): scores[qt,kt] = f32(f64 dot of the tile means,
+ * d ascending from -0.0, times f64(scale)). The device computes the same chain, so block lists compare
+ * bit for bit with the host oracle's (the reference's own device path runs cuBLAS f32 here,
+ * C/rt/vsa.rs:385-388, whose summation order is unspecified). */
 void fvo_vsa_coarse_scores(const float* qc, const float* kc, float* scores, size_t bh, size_t nb,
                            size_t dim, float scale);
 

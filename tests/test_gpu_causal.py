@@ -93,6 +93,40 @@ def test_sq_ne_sk_and_first_block_rows(fv, oracle):
     assert_parity(got[:, :bt].cpu().numpy(), want0, "causal_block0_rows")
 
 
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("bh,sq,sk,bt,win,sink", [
+    (2, 512, 256, 256, 1, 0),     # the second query tile walks no key tile at all
+    (1, 1000, 300, 100, 2, 0),    # rows 500.. see nothing; the tile 256..511 is partly visible
+    (2, 1000, 300, 100, 2, 1),    # same with a sink block: every row sees block 0
+    (1, 700, 130, 64, 0, 0),      # more queries than keys, no window: the late rows see every key
+])
+def test_more_queries_than_keys_with_a_window(fv, oracle, bh, sq, sk, bt, win, sink, d):
+    """sq > sk with a window lets the window slide past the last key: such rows have no visible key and
+    come out as zeros (the reference's kernel runs zero iterations and stores acc * 0,
+    kernels/attn2.cu:214-221, 330-352), whole tiles of them included; every other row matches the
+    masked oracle. The output buffer is poisoned first, so an unwritten row cannot pass."""
+    import torch
+
+    seed = 4100 + sq + d
+    announce(f"causal sq>sk bh={bh} sq={sq} sk={sk} d={d} block={bt} window={win} sink={sink} seed={seed}")
+    q, k, v = qkv(seed, bh, sq, sk, d)
+    tq, tk = np.arange(sq)[:, None] // bt, np.arange(sk)[None, :] // bt
+    vis = (tk < sink) | ((tk <= tq) & ((win == 0) | (tq - tk < win)))
+    live = vis.any(axis=1)
+    assert (win == 0 or sink > 0) == bool(live.all())
+    want = oracle.sdpa_f64(q, k, v, mask_bc=(bt, win, sink), rows=np.nonzero(live)[0])
+    qd, kd, vd = (to_dev_bf16(x) for x in (q, k, v))
+    for out_bf16 in (False, True):
+        out = torch.full((bh, sq, d), float("nan"), device="cuda", dtype=torch.bfloat16 if out_bf16 else torch.float32)
+        fv.sdpa_block_causal_bf16(qd, kd, vd, bt, win, sink, out_bf16=out_bf16, out=out)
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        assert np.isfinite(got).all()
+        assert np.all(got[:, ~live] == 0.0)
+        assert_parity(got[:, live], want, f"causal_sq{sq}_sk{sk}_{bt}_{win}_{sink}_bf16out{int(out_bf16)}",
+                      max_abs=2e-2 if out_bf16 else 1e-2)
+
+
 def test_declines(fv):
     import torch
 

@@ -203,17 +203,15 @@ def test_whole_op_vs_host_oracle(fv, oracle, grid, in_bf16):
     got, sel = fv.vsa_attention_device(cast(q), cast(k), cast(v), cast(g), ctx, float(scale), return_selected=True)
     torch.cuda.synchronize()
     got, sel = got.cpu().numpy(), sel.cpu().numpy().view(np.uint32)
-    # block index lists: bit-exact against the device-order restatement on the same scores
+    # block index lists: the device computes the host oracle's own scores (f64 dot, rt/vsa.rs:185-189),
+    # so it selects the host oracle's tiles, row for row; its list order is the device contract
+    # (above the threshold ascending, then ties ascending; kernels/core.cu:580-618)
+    assert np.array_equal(np.sort(sel, -1), np.sort(want_sel.reshape(sel.shape), -1))
     qc, kc = oracle.vsa_tile_mean(q, oplan), oracle.vsa_tile_mean(k, oplan)
     scores = oracle.vsa_coarse_scores(qc, kc, scale)
     assert np.array_equal(sel, oracle.topk_device_order(scores, ctx.topk).reshape(sel.shape))
-    # and the same SETS as the host oracle's f64-dot selection (ties/near-ties aside)
-    diff = (np.sort(sel, -1) != np.sort(want_sel, -1)).any(-1).sum()
-    print(f"selection rows differing from the f64 host oracle: {diff} of {sel.shape[0] * sel.shape[1]}")
-    m = assert_parity(got, want, f"vsa_op_{grid}_{'bf16' if in_bf16 else 'f32'}", max_abs=1e-2 if diff == 0 else 1.0,
-                      min_cos=0.9999 if diff == 0 else 0.99)
-    if diff == 0:
-        assert m["rel_l2"] <= 2e-2
+    m = assert_parity(got, want, f"vsa_op_{grid}_{'bf16' if in_bf16 else 'f32'}")
+    assert m["rel_l2"] <= 2e-2
     # gate None == gate of ones
     ones = np.ones_like(q)
     a = fv.vsa_attention_device(cast(q), cast(k), cast(v), None, ctx, float(scale))
@@ -290,8 +288,8 @@ def test_declines_and_errors(fv):
 @pytest.mark.parametrize("grid,topk", [((32, 32, 32), 64), ((21, 30, 52), 125)])
 def test_headline_vsa_shapes(fv, oracle, grid, topk):
     """The synthetic VSA benchmark geometry (512 full cubes, top-k 64 of 512) and the reference's own Wan
-    480p geometry (624 tiles, top-k 125), H = 12, bf16: block index lists bit-exact at
-    full size; fine + combine output checked on sampled query tiles."""
+    480p geometry (624 tiles, top-k 125), H = 12, bf16: block index lists equal to the host oracle's at
+    full size (every row of every head); fine + combine output checked on sampled query tiles."""
     import torch
 
     bh = 12
@@ -299,15 +297,17 @@ def test_headline_vsa_shapes(fv, oracle, grid, topk):
     ctx = fv.VsaCtx(grid, 0.8)
     oplan = oracle.TilePlan(grid)
     nb = ctx.num_tiles
-    gen = torch.Generator(device="cuda").manual_seed(99)
-    q, k, v, g = (torch.randn((bh, ctx.seq, D), generator=gen, device="cuda").to(torch.bfloat16) for _ in range(4))
+    qn, kn, vn, gn = (oracle.quantize_bf16(randn(990 + i, (bh, ctx.seq, D))) for i in range(4))
+    q, k, v, g = (dev(x).to(torch.bfloat16) for x in (qn, kn, vn, gn))
     scale = np.float32(1.0 / np.sqrt(D))
     out, sel = fv.vsa_attention_device(q, k, v, g, ctx, float(scale), topk=topk, return_selected=True)
     torch.cuda.synchronize()
-    qn, kn, vn, gn = (x.float().cpu().numpy() for x in (q, k, v, g))
     sel = sel.cpu().numpy().view(np.uint32)
+    # stages 1-3 of the host oracle (rt/vsa.rs:151-212) at full size: tile means, f64-dot scores, top-k
     scores = oracle.vsa_coarse_scores(oracle.vsa_tile_mean(qn, oplan), oracle.vsa_tile_mean(kn, oplan), scale)
-    assert np.array_equal(sel, oracle.topk_device_order(scores, topk).reshape(sel.shape))
+    host_sel = oracle.topk_host_order(scores, topk).reshape(sel.shape)
+    assert np.array_equal(np.sort(sel, -1), np.sort(host_sel, -1))          # the reference's block lists, as sets
+    assert np.array_equal(sel, oracle.topk_device_order(scores, topk).reshape(sel.shape))   # in the device order
     # sampled query tiles: f64 fine attention over the selected tiles + coarse branch
     vc = oracle.vsa_tile_mean(vn, oplan).astype(np.float64)
     rng = np.random.Generator(np.random.PCG64(5))

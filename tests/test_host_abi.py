@@ -109,3 +109,42 @@ def test_dense_route_collapsed():
     for b in ("host", "sparse"):
         assert fv_sdpa.dense_route(*s, backend_name=b) == ["retired"]
         assert fv_sdpa.dense_route(*s, masked=True, backend_name=b) == ["composed"]   # masked calls never look
+
+
+@pytest.mark.parametrize("bt,win,sink,sq,sk", [
+    (256, 1, 0, 512, 256),      # the second query tile sees no key at all
+    (100, 2, 0, 1000, 300), (100, 2, 1, 1000, 300), (64, 0, 0, 700, 130), (1560, 0, 0, 4680, 4680),
+    (1560, 2, 1, 6240, 4680), (7, 3, 2, 900, 200), (300, 1, 0, 2000, 500), (128, 1, 3, 1024, 4096),
+    (50, 4, 0, 257, 1), (1000, 1, 0, 513, 64)])
+def test_block_causal_tile_walk_covers_every_visible_key(bt, win, sink, sq, sk):
+    """The key-tile ranges the fused block-causal kernel walks (the function the kernel itself runs):
+    ascending, disjoint, inside the key tiles, and covering every key that rt/attn.rs:449-453 lets any
+    query of the tile see; a tile whose walk is empty has no visible key at all."""
+    lib = fv_sdpa.lib()
+    nkt = (sk + 63) // 64
+    q = np.arange(sq)[:, None]
+    k = np.arange(sk)[None, :]
+    tq, tk = q // bt, k // bt
+    vis = (tk < sink) | ((tk <= tq) & ((win == 0) | (tq - tk < win)))
+    empty_tiles = 0
+    for q0 in range(0, sq, 256):
+        out = (ctypes.c_int * 4)()
+        assert lib.fv_block_causal_tile_walk(bt, win, sink, sq, sk, q0, out) == 0
+        n0, a1, n1, total = list(out)
+        assert 0 <= n0 <= a1 and n1 >= 0 and a1 + n1 <= nkt and total == n0 + n1
+        walked = np.zeros(nkt, bool)
+        walked[:n0] = True
+        walked[a1:a1 + n1] = True
+        need = vis[q0:q0 + 256].any(axis=0)                       # keys some query of the tile sees
+        need_tiles = np.zeros(nkt, bool)
+        need_tiles[np.nonzero(need)[0] // 64] = True
+        assert not (need_tiles & ~walked).any(), (q0, list(out))
+        if total == 0:
+            assert not need.any()
+            empty_tiles += 1
+    if (bt, win, sink, sq, sk) == (256, 1, 0, 512, 256):
+        assert empty_tiles == 1
+    # parameters the kernel declines
+    out = (ctypes.c_int * 4)()
+    assert lib.fv_block_causal_tile_walk(0, 0, 0, 256, 256, 0, out) == _lib.FV_DECLINED
+    assert lib.fv_block_causal_tile_walk(64, 0, 0, 256, 256, 100, out) == _lib.FV_DECLINED

@@ -234,13 +234,45 @@ def test_combine_forms(oracle):
     assert np.all(out[:, ~inside] == 7.0) and np.all(out[:, inside] != 7.0)
 
 
-def test_coarse_scores_vs_f64(oracle):
+def test_coarse_scores_are_the_sequential_f64_dot(oracle):
+    # C/rt/vsa.rs:185-189: f64 products summed in ascending d, times f64(scale), one rounding to f32
     rng = np.random.default_rng(3)
     qc = rng.standard_normal((2, 9, 128)).astype(np.float32)
     kc = rng.standard_normal((2, 9, 128)).astype(np.float32)
-    got = oracle.vsa_coarse_scores(qc, kc, 0.25)
-    want = np.einsum("bqd,bkd->bqk", qc.astype(np.float64), kc.astype(np.float64)) * 0.25
-    assert np.abs(got - want).max() < 1e-5
+    scale = np.float32(0.25 / 3)
+    got = oracle.vsa_coarse_scores(qc, kc, scale)
+    prod = qc.astype(np.float64)[:, :, None, :] * kc.astype(np.float64)[:, None, :, :]
+    dot = np.cumsum(prod, axis=-1)[..., -1]          # cumsum adds strictly left to right
+    want = (dot * np.float64(scale)).astype(np.float32)
+    assert np.array_equal(got, want)
+    # an f32 accumulation of the same products differs in some last bits: the test can tell the two apart
+    f32 = np.zeros((2, 9, 9), np.float32)
+    for d in range(128):
+        f32 = f32 + qc[:, :, None, d] * kc[:, None, :, d]
+    assert np.any(f32 * scale != got)
+
+
+def test_coarse_scores_zero_signs(oracle):
+    # the sum starts from -0.0 (Rust's f64 Sum identity): products that are all -0.0 give -0.0,
+    # any +0.0 among them gives +0.0
+    qc = np.zeros((1, 2, 4), np.float32)
+    kc = np.array([[[1, 2, 3, 4], [-1, -2, -3, -4]]], np.float32)
+    got = oracle.vsa_coarse_scores(qc, kc, 0.5)
+    assert np.all(got == 0) and not np.signbit(got[0, 0, 0]) and np.signbit(got[0, 0, 1])
+    kc[0, 1, 2] = 3.0
+    assert not np.signbit(oracle.vsa_coarse_scores(qc, kc, 0.5)[0, 0, 1])
+
+
+def test_coarse_scores_are_what_the_host_oracle_selects_from(oracle):
+    # stage 3 of vsa_attention_host sorts exactly these scores (C/rt/vsa.rs:203-212)
+    plan = oracle.TilePlan((5, 6, 7))
+    rng = np.random.default_rng(8)
+    q, k, v = (rng.standard_normal((2, plan.seq, 16)).astype(np.float32) for _ in range(3))
+    scale = 0.25
+    topk = 3
+    _, sel = oracle.vsa_attention_host(q, k, v, None, plan, topk, 1, 2, 16, scale, return_selected=True)
+    sc = oracle.vsa_coarse_scores(oracle.vsa_tile_mean(q, plan), oracle.vsa_tile_mean(k, plan), scale)
+    assert np.array_equal(sel.reshape(-1, topk), oracle.topk_host_order(sc, topk))
 
 
 # ---- VSA host oracle -----------------------------------------------------------------------
