@@ -8,9 +8,8 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache|kvcache1|composed|
-softmax|machine) are for the design notes; the driver's line is the default `self`. `machine` measures the box, not
-the library: the rate of an MFMA-only loop at several launch lengths and of a plain copy.
+Other workloads (--workload cross|causal|causal3|c5|c5cross|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache|kvcache1|
+composed|softmax) are for the design notes; the driver's line is the default `self`.
 """
 import argparse
 import json
@@ -24,9 +23,10 @@ sys.path.insert(0, os.path.join(ROOT, "fastvideo-rs_amd"))
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the flash kernel at the headline workload, from two counter runs
-# (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, factors from a plain 1 GiB copy in the same runs).
-MEASURED_TRAFFIC_BYTES = {"self": 1.0065e9}
+# HBM bytes per launch of the flash kernel at the headline workload. NOT measured by this script: the figure
+# comes from two rocprofv3 --pmc runs of this same command (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, the
+# factors from a plain 1 GiB copy in the same runs), whose summary is the file named beside it.
+MEASURED_TRAFFIC_BYTES = {"self": (1.0065e9, "profiles/flash_fwd_pp2_wan13b_self_attention.md")}
 
 WORKLOADS = {
     # name: (H, Sq, Sk, causal block_tokens or 0, description)
@@ -387,91 +387,6 @@ def bench_softmax(args):
     print(json.dumps(rec), flush=True)
 
 
-def bench_machine(args):
-    """What this box gives a kernel with nothing in its way: an MFMA-only loop (bf16 32x32x16, register
-    operands, 2 waves per SIMD on every CU) at launch lengths from tens of microseconds to tens of
-    milliseconds, and a plain 1 GiB copy. The long launches show the clock the chip holds under matrix
-    load; their rate is the ceiling an MFMA-bound kernel sees here."""
-    import ctypes as C
-
-    import torch
-
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    path = os.path.join(ROOT, "fastvideo-rs_amd", "libfv_probes.so")
-    if not os.path.exists(path):
-        print(f"bench.py: {path} is not built (make -C fastvideo-rs_amd/csrc)", file=sys.stderr)
-        sys.exit(4)
-    lib = C.CDLL(path)
-    lib.fv_probe_mfma_bf16.restype = C.c_int
-    lib.fv_probe_mfma_bf16.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.c_void_p]
-    lib.fv_probe_copy_f32x4.restype = C.c_int
-    lib.fv_probe_copy_f32x4.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
-    stream = torch.cuda.current_stream().cuda_stream
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    blocks = 2 * cus
-    sink = torch.empty(blocks * 256, device=dev)
-    flops = C.c_double()
-    mfma = []
-    for pattern in (0, 1):
-        for iters in (64, 1024, 8192, 65536, 262144):
-            for rep in range(3):    # the last repetition is the one reported
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                rc = lib.fv_probe_mfma_bf16(sink.data_ptr(), blocks, iters, pattern, C.byref(flops), stream)
-                b.record()
-                torch.cuda.synchronize()
-                if rc != 0:
-                    raise RuntimeError(f"fv_probe_mfma_bf16 rc={rc}")
-            ms = a.elapsed_time(b)
-            tf = flops.value / ms / 1e9
-            # 4 SIMDs per CU, one 32x32x16 MFMA (32768 FLOP) per 32 cycles per SIMD when the pipe never idles
-            mfma.append({"operands": "random" if pattern else "constant", "iters": iters, "ms": round(ms, 4),
-                         "TFLOPs": round(tf, 1), "implied_clock_GHz": round(tf * 1e12 / (cus * 4 * 1024) / 1e9, 3)})
-    # the block-sparse fine kernel's load pattern alone: 16 KB tiles through LDS-DMA, 4 workgroups per CU
-    lib.fv_probe_tile_dma.restype = C.c_int
-    lib.fv_probe_tile_dma.argtypes = [C.c_void_p, C.c_uint, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double), C.c_void_p]
-    tiles_buf = torch.zeros(2 << 30, dtype=torch.uint8, device=dev)
-    nbytes = C.c_double()
-    dma = []
-    for region_tiles in (64, 4096, 131072):
-        for rep in range(3):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            rc = lib.fv_probe_tile_dma(tiles_buf.data_ptr(), region_tiles, 4 * cus, 1000, None, C.byref(nbytes), stream)
-            b.record()
-            torch.cuda.synchronize()
-            if rc != 0:
-                raise RuntimeError(f"fv_probe_tile_dma rc={rc}")
-        ms = a.elapsed_time(b)
-        dma.append({"region_MiB": region_tiles * 16 // 1024, "ms": round(ms, 4), "TBps": round(nbytes.value / ms / 1e9, 2)})
-    del tiles_buf
-    n = 1 << 30
-    src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
-    dst = torch.empty_like(src)
-    for rep in range(3):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        rc = lib.fv_probe_copy_f32x4(src.data_ptr(), dst.data_ptr(), n // 16, 16 * cus, stream)
-        b.record()
-        torch.cuda.synchronize()
-        if rc != 0:
-            raise RuntimeError(f"fv_probe_copy_f32x4 rc={rc}")
-    copy_ms = a.elapsed_time(b)
-    copy_gbs = 2.0 * n / copy_ms / 1e6
-    long_run = mfma[-1]
-    rec = {
-        "metric": "MFMA-only bf16 TFLOP/s sustained on this box, random operands (not a library kernel)", "value": long_run["TFLOPs"],
-        "unit": "TFLOP/s", "n_gpus": 1, "steps": 1, "warmup": 2, "ms_per_step": long_run["ms"], "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "machine probe: v_mfma_f32_32x32x16_bf16 loop, 2 waves per SIMD; 1 GiB copy", "cus": cus,
-                   "mfma_only": mfma, "tile_dma_only": dma, "copy_1GiB": {"ms": round(copy_ms, 4), "GBps_read_plus_write": round(copy_gbs, 1)}},
-        "roofline": {"bound": "mfma", "achieved": long_run["TFLOPs"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(long_run["TFLOPs"] / PEAK_BF16_TFLOPS, 4), "traffic": None},
-    }
-    print(json.dumps(rec), flush=True)
-
-
 def visible_pairs(sq, sk, bt):
     if bt == 0:
         return sq * sk
@@ -493,8 +408,9 @@ def visible_pairs(sq, sk, bt):
     return total
 
 
-def cpu_baseline(h, sq, sk, d, bt, flops_full, q, k, v, budget_s):
-    """Time the oracle's fp32 composed SDPA on a bounded sample of query rows."""
+def cpu_baseline(h, sq, sk, d, bt, flops_full, q, k, v, budget_s, gpu_out=None):
+    """Time the oracle's fp32 composed SDPA on a bounded sample of query rows; with `gpu_out` (the
+    kernel's output of the timed launches) also compare those rows, all heads, with the oracle's."""
     import numpy as np
 
     import oracle
@@ -508,15 +424,26 @@ def cpu_baseline(h, sq, sk, d, bt, flops_full, q, k, v, budget_s):
     def run(n):
         rows = np.sort(rng.choice(sq, size=min(n, sq), replace=False)).astype(np.int64)
         t0 = time.perf_counter()
-        oracle.sdpa_composed_rows(qn, kn, vn, rows, mask_bc=mask, threads=threads)
-        return time.perf_counter() - t0, rows.size
+        want = oracle.sdpa_composed_rows(qn, kn, vn, rows, mask_bc=mask, threads=threads)
+        return time.perf_counter() - t0, rows, want
 
-    t_probe, n_probe = run(min(16, sq))
-    per_row = max(t_probe / n_probe, 1e-9)
-    n = int(max(n_probe, min(sq, budget_s / per_row)))
-    t, n = run(n)
+    t_probe, rows, _ = run(min(16, sq))
+    per_row = max(t_probe / rows.size, 1e-9)
+    t, rows, want = run(int(max(rows.size, min(sq, budget_s / per_row))))
+    n = rows.size
     t_full = t * sq / n
-    return {
+    parity = None
+    if gpu_out is not None:
+        import torch
+
+        got = gpu_out[:, torch.from_numpy(rows).to(gpu_out.device)].float().cpu().numpy().astype(np.float64)
+        w64 = want.astype(np.float64)
+        parity = {"rows": int(n), "heads": int(h), "max_abs": float(np.abs(got - w64).max()),
+                  "cosine": float((got.ravel() @ w64.ravel()) / (np.linalg.norm(got) * np.linalg.norm(w64))),
+                  "tolerance": "max_abs <= 1e-2, cosine >= 0.9999 vs the fp32 host-math oracle",
+                  "finite": bool(np.isfinite(got).all())}
+        parity["ok"] = bool(parity["finite"] and parity["max_abs"] <= 1e-2 and parity["cosine"] >= 0.9999)
+    return parity, {
         "value": flops_full / t_full / 1e12,
         "unit": "TFLOP/s",
         "cores": threads,
@@ -534,7 +461,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=8,
                     help="untimed launches first; the shader clock under this kernel takes about six launches to settle")
-    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "kvcache1", "composed", "softmax", "machine"])
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "kvcache1", "composed", "softmax"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
     ap.add_argument("--inputs", default="randn", choices=["randn", "zeros"],
@@ -570,9 +497,6 @@ def main():
         return
     if args.workload == "softmax":
         bench_softmax(args)
-        return
-    if args.workload == "machine":
-        bench_machine(args)
         return
     fv_sdpa.lib()
     dev = torch.device("cuda:0")
@@ -632,6 +556,9 @@ def main():
     achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
     bytes_min = 2.0 * (2 * h * sq * d + 2 * h * sk * d)
 
+    traffic, traffic_source = MEASURED_TRAFFIC_BYTES.get(args.workload, (None, None)) if args.out_bf16 else (None, None)
+    if traffic_source:
+        traffic_source += " (rocprofv3 --pmc runs of this command; not measured in this run)"
     rec = {
         "metric": "SDPA TFLOP/s + % bf16 MFMA peak, Wan-1.3B 480p self-attn (S=32760,H=12,d=128)"
         if args.workload == "self" else f"SDPA TFLOP/s ({args.workload})",
@@ -652,15 +579,22 @@ def main():
         "pct_of_bf16_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.out_bf16 else None,
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": f"fv::flash_fwd_pp2<{'true' if bt else 'false'}, {d}>",
                      "avg_kernel_ms": round(avg_kernel_ms, 4), "median_kernel_ms": round(kern_ms[len(kern_ms) // 2], 4),
                      "min_hbm_bytes": bytes_min,
                      "hbm_frac_at_min_traffic": round(bytes_min / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
     }
     if args.cpu_seconds > 0 and bt >= 0:   # the row-sampled oracle takes dense and block-causal masks
-        rec["cpu_baseline"] = cpu_baseline(h, sq, sk, d, bt, flops, q, k, v, args.cpu_seconds)
+        # outside the timed region; the rows the baseline computes double as a parity sample of this run's output
+        parity, rec["cpu_baseline"] = cpu_baseline(h, sq, sk, d, bt, flops, q, k, v, args.cpu_seconds,
+                                                   out if args.inputs == "randn" else None)
+        if parity is not None:
+            rec["parity"] = parity
     print(json.dumps(rec), flush=True)
+    if rec.get("parity") is not None and not rec["parity"]["ok"]:
+        print("bench.py: the timed launches' output is outside the parity tolerance", file=sys.stderr)
+        sys.exit(5)
 
 
 if __name__ == "__main__":

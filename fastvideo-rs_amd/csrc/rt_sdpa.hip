@@ -149,7 +149,7 @@ Result<const Tensor*> as_bf16(const Tensor& x, Tensor& tmp, hipStream_t st) {
     if (!is_ok(r)) return std::get<TensorError>(r);
     tmp = std::move(std::get<Tensor>(r));
     const int rc = fv_cast_f32_bf16((const float*)x.data, (uint16_t*)tmp.data, x.numel(), st);
-    if (rc != FV_OK) return msg("cast_f32_bf16: " + rc_message(rc));
+    if (rc != FV_OK) return TensorError{"cast_f32_bf16: " + rc_message(rc), rc < 0 ? -rc : 0};
     g_cast++;
     return &tmp;
 }
@@ -160,7 +160,7 @@ Result<const Tensor*> as_f32(const Tensor& x, Tensor& tmp, hipStream_t st) {
     if (!is_ok(r)) return std::get<TensorError>(r);
     tmp = std::move(std::get<Tensor>(r));
     const int rc = fv_cast_bf16_f32((const uint16_t*)x.data, (float*)tmp.data, x.numel(), st);
-    if (rc != FV_OK) return msg("cast_bf16_f32: " + rc_message(rc));
+    if (rc != FV_OK) return TensorError{"cast_bf16_f32: " + rc_message(rc), rc < 0 ? -rc : 0};
     g_cast++;
     return &tmp;
 }
@@ -199,7 +199,8 @@ Result<Tensor> compact(const Tensor& x, hipStream_t st) {
     if (planes && x.shape[2] && row) {
         const hipError_t e = hipMemcpy2DAsync(t.data, x.shape[2] * row, x.data, x.plane_rows * row, x.shape[2] * row,
                                               planes, hipMemcpyDeviceToDevice, st);
-        if (e != hipSuccess) return msg(std::string("sdpa: compacting a row window: ") + hipGetErrorString(e));
+        if (e != hipSuccess)
+            return TensorError{std::string("sdpa: compacting a row window: ") + hipGetErrorString(e), (int)e};
     }
     return std::move(t);
 }
@@ -251,7 +252,7 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
         }
     }
     if (rc == FV_DECLINED) return std::optional<Tensor>{};
-    if (rc != FV_OK) return msg("sdpa: " + rc_message(rc));
+    if (rc != FV_OK) return TensorError{"sdpa: " + rc_message(rc), rc < 0 ? -rc : 0};
     ((causal || window) ? g_causal : g_fused)++;
     return std::optional<Tensor>{std::move(out)};
 }
@@ -399,7 +400,10 @@ Result<Tensor> Tensor::alloc(std::vector<size_t> shape, DType dtype, hipStream_t
     t.dtype = dtype;
     const size_t bytes = (t.numel() ? t.numel() : 1) * elem_size(dtype);
     hipError_t e = hipMallocAsync(&t.data, bytes, stream);
-    if (e != hipSuccess) return msg(std::string("sdpa: device allocation failed: ") + hipGetErrorString(e));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();   // the failed allocation is reported here, not by the next launch
+        return TensorError{std::string("sdpa: device allocation failed: ") + hipGetErrorString(e), (int)e};
+    }
     t.owned_ = true;
     t.stream_ = stream;
     return std::move(t);
@@ -564,6 +568,8 @@ Result<Tensor> sdpa_composed(const Tensor& q, const Tensor& k, const Tensor& v, 
         const size_t r = mask->rank();
         if (r < 2 || mask->shape[r - 2] != sq || mask->shape[r - 1] != sk)
             return msg("sdpa: mask must be [.., sq, sk]");
+        if (sq == 0) return Tensor::alloc({b, h, 0, d}, DType::F32, st);   // no query rows: an empty result
+        if (sk == 0) return msg("sdpa: no keys");
         const size_t lead = mask->numel() / (sq * sk);
         if (lead == b * h && lead != 1) mask_per_bh = 1;
         else if (lead != 1) return msg("sdpa: mask batch must be 1 or batch*heads");
@@ -587,7 +593,7 @@ Result<Tensor> sdpa_composed(const Tensor& q, const Tensor& k, const Tensor& v, 
                                         pm ? (const float*)pm->data : nullptr, mask_per_bh, (float*)out.data, b * h,
                                         sq, sk, d, default_scale(scale, d), st);
     if (rc == FV_DECLINED) return msg("sdpa: every kernel of the route declined");
-    if (rc != FV_OK) return msg("sdpa: " + rc_message(rc));
+    if (rc != FV_OK) return TensorError{"sdpa: " + rc_message(rc), -rc};
     g_composed++;
     return std::move(out);
 }
@@ -677,7 +683,12 @@ int fv_rt_sdpa(const fv_tensor* q, const fv_tensor* k, const fv_tensor* v, const
             return fv_invalid("fv_rt_sdpa: unknown plan kind");
     }
     auto r = sdpa(tq, tk, tv, p, (hipStream_t)stream);
-    if (!is_ok(r)) return fv_invalid(std::get<TensorError>(r).message.c_str());
+    if (!is_ok(r)) {
+        // a refused argument is -hipErrorInvalidValue; an allocation or launch failure keeps its own code
+        const TensorError& err = std::get<TensorError>(r);
+        const int rc = fv_invalid(err.message.c_str());
+        return err.hip_code > 0 ? -err.hip_code : rc;
+    }
     Tensor& t = std::get<Tensor>(r);
     out->rank = (int)t.rank();
     for (size_t i = 0; i < t.rank() && i < 8; i++) out->shape[i] = t.shape[i];

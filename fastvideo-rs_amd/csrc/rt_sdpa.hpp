@@ -23,6 +23,7 @@ enum class DType : int { F32 = 0, Bf16 = 1 };
 // rt/tensor.rs:92-98 `TensorError::Message`
 struct TensorError {
     std::string message;
+    int hip_code = 0;   // the hipError_t behind the message (allocation, launch); 0 = a refused argument
 };
 
 template <class T>

@@ -14,7 +14,12 @@ __all__ = ["Plan", "BlockCausal", "VdnWindow", "sdpa", "with_bf16_act", "bf16_ac
 
 
 class TensorError(RuntimeError):
-    """rt/tensor.rs:92-98 `TensorError::Message`."""
+    """rt/tensor.rs:92-98 `TensorError::Message`. `rc` is the C ABI's return: -hipErrorInvalidValue (-1) for a
+    refused argument, the negated hipError_t of a failed allocation (-2 out of memory) or launch otherwise."""
+
+    def __init__(self, message, rc=None):
+        super().__init__(message)
+        self.rc = rc
 
 
 class _FvTensor(C.Structure):
@@ -177,7 +182,7 @@ def sdpa(q, k, v, plan):
     stream = torch.cuda.current_stream().cuda_stream
     rc = lib.fv_rt_sdpa(C.byref(dq), C.byref(dk), C.byref(dv), C.byref(p), C.byref(out), stream)
     if rc != 0:
-        raise TensorError(lib.fv_sdpa_last_error().decode())
+        raise TensorError(lib.fv_sdpa_last_error().decode(), rc)
     shape = tuple(out.shape[i] for i in range(out.rank))
     dtype = torch.bfloat16 if out.dtype else torch.float32
     n = 1

@@ -137,20 +137,22 @@ def test_declines(fv):
 
 @pytest.mark.parametrize("bt", [1560, 4680])
 def test_headline_causal_shape_sampled_rows(fv, oracle, bt):
-    """Self-Forcing frame-causal at full size (21 frames x 1560 tokens) and the
-    reference's own 3-frame blocks; parity on sampled rows incl. frame edges."""
+    """Self-Forcing frame-causal at full size (21 frames x 1560 tokens) and the reference's own 3-frame
+    blocks, inputs from numpy's PCG64: parity of every head on more than 512 query rows, the last row of
+    every block and the first row of the next among them (both sides of every mask boundary)."""
     import torch
 
     bh, s, d = 12, 32760, 128
-    announce(f"causal headline bh={bh} s={s} block={bt}")
-    g = torch.Generator(device="cuda").manual_seed(77)
-    q, k, v = (torch.randn((bh, s, d), generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    announce(f"causal headline bh={bh} s={s} block={bt} seed=77")
+    qn, kn, vn = qkv(77, bh, s, s, d)
+    q, k, v = (to_dev_bf16(x) for x in (qn, kn, vn))
     out = fv.sdpa_block_causal_bf16(q, k, v, bt, 0, 0)
     torch.cuda.synchronize()
-    rows = sample_rows(3, s, 24, extra=(0, bt - 1, bt, 2 * bt - 1, 2 * bt, 10 * bt + 5, s - bt, s - 1))
-    want = oracle.sdpa_composed_rows(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), rows,
-                                     mask_bc=(bt, 0, 0))
-    assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, f"causal_headline_{bt}")
+    edges = [e for b in range(bt, s, bt) for e in (b - 1, b)]
+    rows = sample_rows(3, s, 512, extra=[0, 255, 256, 10 * bt + 5, s - 1] + edges)
+    assert rows.size >= 512 and set(edges) <= set(rows.tolist())
+    want = oracle.sdpa_composed_rows(qn, kn, vn, rows, mask_bc=(bt, 0, 0))
+    assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, f"causal_headline_{bt}_{rows.size}_rows")
     # the bf16 output is the RNE rounding of the f32 output, every element
     assert torch.equal(fv.sdpa_block_causal_bf16(q, k, v, bt, 0, 0, out_bf16=True), out.to(torch.bfloat16))
 

@@ -172,32 +172,39 @@ def test_declines(fv):
 
 
 def test_headline_shape_sampled_rows(fv, oracle):
-    """Wan-1.3B 480p self-attention at full size: S = 32760, H = 12; parity on sampled rows."""
+    """Wan-1.3B 480p self-attention at full size (S = 32760, H = 12), inputs from numpy's PCG64: parity of
+    every head on more than 1024 query rows, the first and last row of several 256-query workgroup tiles
+    and of the last, partial one included; the same rows against the 512-key cross-attention call."""
     import torch
 
     bh, s, d = 12, 32760, 128
-    announce(f"dense headline bh={bh} s={s}")
-    g = torch.Generator(device="cuda").manual_seed(2024)
-    q, k, v = (torch.randn((bh, s, d), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3))
+    announce(f"dense headline bh={bh} s={s} seed=2024")
+    qn, kn, vn = qkv(2024, bh, s, s, d)
+    q, k, v = (to_dev_bf16(x) for x in (qn, kn, vn))
     out = fv.sdpa_dense_bf16(q, k, v)
     torch.cuda.synchronize()
-    rows = sample_rows(1, s, 48, extra=(0, 127, 128, s - 1, s - 57))
-    want = oracle.sdpa_composed_rows(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), rows)
-    assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, "dense_headline_rows")
+    last_tile = (s - 1) // 256 * 256
+    rows = sample_rows(1, s, 1024, extra=(0, 31, 32, 127, 128, 255, 256, 511, 512, 16383, 16384, last_tile - 1, last_tile,
+                                          last_tile + 31, last_tile + 32, s - 57, s - 1))
+    assert rows.size >= 1024
+    ridx = torch.from_numpy(rows).cuda()
+    want = oracle.sdpa_composed_rows(qn, kn, vn, rows)
+    assert_parity(out[:, ridx].cpu().numpy(), want, f"dense_headline_{rows.size}_rows_x_{bh}_heads")
     # cross-attention: same queries against 512 keys
     kc, vc = k[:, :512].contiguous(), v[:, :512].contiguous()
     outc = fv.sdpa_dense_bf16(q, kc, vc)
     torch.cuda.synchronize()
-    wantc = oracle.sdpa_composed_rows(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), rows)
-    assert_parity(outc[:, torch.from_numpy(rows).cuda()].cpu().numpy(), wantc, "cross_headline_rows")
+    wantc = oracle.sdpa_composed_rows(qn, np.ascontiguousarray(kn[:, :512]), np.ascontiguousarray(vn[:, :512]), rows)
+    assert_parity(outc[:, ridx].cpu().numpy(), wantc, f"cross_headline_{rows.size}_rows_x_{bh}_heads")
     # the bf16 output (whole rows staged through LDS) is the RNE rounding of the f32 output, every element
     assert torch.equal(fv.sdpa_dense_bf16(q, k, v, out_bf16=True), out.to(torch.bfloat16))
     assert torch.equal(fv.sdpa_dense_bf16(q, kc, vc, out_bf16=True), outc.to(torch.bfloat16))
 
 
 def test_wan14b_shape_sampled_rows(fv, oracle):
-    """Wan-14B 720p self- and cross-attention at full size (H = 40, S = 75600, Sk = 512): parity on
-    sampled rows; the whole sequence of every head is resident on the one GPU."""
+    """Wan-14B 720p self- and cross-attention at full size (H = 40, S = 75600, Sk = 512): parity of all 40
+    heads on more than 256 query rows incl. workgroup-tile edges; the whole sequence of every head is
+    resident on the one GPU. (Inputs are drawn on the device: 1.2e9 normals; the oracle sees the same values.)"""
     import torch
 
     bh, s, d = 40, 75600, 128
@@ -206,17 +213,18 @@ def test_wan14b_shape_sampled_rows(fv, oracle):
     q, k, v = (torch.randn((bh, s, d), generator=g, device="cuda", dtype=torch.bfloat16) for _ in range(3))
     out = fv.sdpa_dense_bf16(q, k, v, out_bf16=True)
     torch.cuda.synchronize()
-    rows = sample_rows(5, s, 12, extra=(0, 255, 256, s - 1))
+    last_tile = (s - 1) // 256 * 256
+    rows = sample_rows(5, s, 256, extra=(0, 255, 256, 37887, 37888, last_tile - 1, last_tile, s - 1))
+    assert rows.size >= 256
     ridx = torch.from_numpy(rows).cuda()
-    heads = [0, 7, 19, 39]      # the oracle walks 75600 keys per row: four heads keep it in seconds
-    hk = lambda x: x[heads].float().cpu().numpy()  # noqa: E731
-    want = oracle.sdpa_composed_rows(hk(q), hk(k), hk(v), rows)
-    assert_parity(out[heads][:, ridx].float().cpu().numpy(), want, "wan14b_self_rows", max_abs=2e-2)
+    qn, kn, vn = (x.float().cpu().numpy() for x in (q, k, v))
+    want = oracle.sdpa_composed_rows(qn, kn, vn, rows)
+    assert_parity(out[:, ridx].float().cpu().numpy(), want, f"wan14b_self_{rows.size}_rows_x_{bh}_heads", max_abs=2e-2)
     kc, vc = k[:, :512].contiguous(), v[:, :512].contiguous()
     outc = fv.sdpa_dense_bf16(q, kc, vc)
     torch.cuda.synchronize()
-    wantc = oracle.sdpa_composed_rows(hk(q), hk(kc), hk(vc), rows)
-    assert_parity(outc[heads][:, ridx].cpu().numpy(), wantc, "wan14b_cross_rows")
+    wantc = oracle.sdpa_composed_rows(qn, np.ascontiguousarray(kn[:, :512]), np.ascontiguousarray(vn[:, :512]), rows)
+    assert_parity(outc[:, ridx].cpu().numpy(), wantc, f"wan14b_cross_{rows.size}_rows_x_{bh}_heads")
 
 
 @pytest.mark.parametrize("bh,s", [(12, 32760), (40, 75600)])

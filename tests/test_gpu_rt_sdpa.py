@@ -221,3 +221,37 @@ def test_composed_kernel_vs_oracle(fv, oracle, bh, sq, sk, d, mask_kind):
     m = metrics(host(out), want)
     print(m)
     assert m["max_abs"] < 2e-5
+
+
+def test_allocation_failure_is_reported_with_its_own_code_and_leaves_the_device_usable(fv):
+    """A result larger than the device's memory: `sdpa` fails at its first allocation, before any
+    launch (the operand descriptors claim 130 M query rows; nothing ever reads them), with the
+    out-of-memory code rather than the code of a refused argument, and the next call works."""
+    import ctypes
+    import torch
+
+    from fv_sdpa.sdpa import _FvPlan, _FvTensor
+
+    announce("rt allocation failure, 12 x 130e6 x 128 bf16 result (400 GB)")
+    buf = torch.zeros((1, 12, 256, 128), device="cuda", dtype=torch.bfloat16)
+
+    def desc(rows):
+        t = _FvTensor()
+        t.data, t.dtype, t.rank, t.plane_rows = buf.data_ptr(), 1, 4, 0
+        for i, s in enumerate((1, 12, rows, 128)):
+            t.shape[i] = s
+        return t
+
+    lib = fv.lib()
+    p = _FvPlan()
+    p.kind, p.kv_flash = 0, -1
+    out = _FvTensor()
+    q, kv = desc(130_000_000), desc(256)
+    rc = lib.fv_rt_sdpa(ctypes.byref(q), ctypes.byref(kv), ctypes.byref(kv), ctypes.byref(p), ctypes.byref(out),
+                        torch.cuda.current_stream().cuda_stream)
+    msg = lib.fv_sdpa_last_error().decode()
+    print(f"rc={rc} message={msg!r}")
+    assert rc == -2 and msg.startswith("sdpa: device allocation failed: ")      # hipErrorOutOfMemory
+    got = fv.sdpa(buf, buf, buf, fv.Plan.dense(None))
+    torch.cuda.synchronize()
+    assert got.shape == buf.shape and torch.isfinite(got.float()).all()

@@ -148,3 +148,59 @@ def test_block_causal_tile_walk_covers_every_visible_key(bt, win, sink, sq, sk):
     out = (ctypes.c_int * 4)()
     assert lib.fv_block_causal_tile_walk(0, 0, 0, 256, 256, 0, out) == _lib.FV_DECLINED
     assert lib.fv_block_causal_tile_walk(64, 0, 0, 256, 256, 100, out) == _lib.FV_DECLINED
+
+
+def _fake_tensor(shape, bf16, addr=0x1000):
+    """A descriptor whose pointer is never dereferenced on the host: for calls that must fail before a launch."""
+    from fv_sdpa.sdpa import _FvTensor
+
+    t = _FvTensor()
+    t.data, t.dtype, t.rank, t.plane_rows = addr, int(bf16), len(shape), 0
+    for i, s in enumerate(shape):
+        t.shape[i] = s
+    return t
+
+
+def _rt_call(q, k, v, kind=0, mask=None):
+    from fv_sdpa.sdpa import _FvPlan, _FvTensor
+
+    lib = fv_sdpa.lib()
+    p = _FvPlan()
+    p.kind, p.kv_flash = kind, -1
+    if mask is not None:
+        p.mask = ctypes.pointer(mask)
+    out = _FvTensor()
+    rc = lib.fv_rt_sdpa(ctypes.byref(q), ctypes.byref(k), ctypes.byref(v), ctypes.byref(p), ctypes.byref(out), None)
+    return rc, lib.fv_sdpa_last_error().decode()
+
+
+def test_rt_sdpa_refuses_before_any_device_work():
+    """Argument errors of the one entry are host decisions: they come back as -hipErrorInvalidValue with the
+    reference's message and touch no device (rt/sdpa.rs:141-164, rt/tensor.rs:1655-1667)."""
+    q = _fake_tensor((1, 2, 8, 128), True)
+    rc, msg = _rt_call(_fake_tensor((2, 8, 128), True), q, q)
+    assert rc == -1 and msg == "sdpa expects BHSD"
+    # a masked composed call with no keys: refused, and the mask's batch count is never divided by sq * sk = 0
+    k0 = _fake_tensor((1, 2, 0, 128), False)
+    rc, msg = _rt_call(_fake_tensor((1, 2, 8, 128), False), k0, k0, kind=1, mask=_fake_tensor((8, 0), False))
+    assert rc == -1 and msg == "sdpa: no keys"
+    rc, msg = _rt_call(q, q, q, kind=99)
+    assert rc == -1 and "unknown plan kind" in msg
+
+
+def test_rt_sdpa_reports_an_allocation_failure_with_its_own_code():
+    """Without a device the first allocation fails: the entry returns that hipError_t (not the code of a
+    refused argument) and the message says which step failed. Skipped where a GPU is present (the
+    allocation would succeed and the fake operands must never reach a kernel)."""
+    import torch
+
+    if torch.cuda.device_count() > 0:
+        pytest.skip("needs a host without a GPU")
+    q = _fake_tensor((1, 2, 8, 128), True)
+    rc, msg = _rt_call(q, q, q)
+    assert rc < -1 and msg.startswith("sdpa: device allocation failed: ")
+    # no query rows + a mask: an empty result is allocated (no division by sq * sk = 0 on the way)
+    q0 = _fake_tensor((1, 2, 0, 128), False)
+    kv = _fake_tensor((1, 2, 8, 128), False)
+    rc, msg = _rt_call(q0, kv, kv, kind=1, mask=_fake_tensor((0, 8), False))
+    assert rc < -1 and msg.startswith("sdpa: device allocation failed: ")
