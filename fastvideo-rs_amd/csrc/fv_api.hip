@@ -5,6 +5,7 @@
 #include <limits.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <string>
 
 #include "fv_common.h"
@@ -49,6 +50,34 @@ __global__ void cast_bf16_f32_kernel(const uint16_t* __restrict__ x, float* __re
                                      size_t n) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) y[i] = fv::bf16_bits_to_f32(x[i]);
+}
+
+// ---- static split-KV buffer ------------------------------------------------------------------
+// The partials of fv_sdpa_dense_bf16_splitkv_static: part of the code object, so every GPU the
+// library runs on holds its own copy at its own address from module load to process end. In host
+// code the array's NAME is only a handle for hipGetSymbolAddress, never a device address: kernels
+// and copies get the per-device pointer resolved below.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// This device's address of `scratch` (resolved once per device, with that device current).
+hipError_t static_scratch(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p || (((uintptr_t)p) & 255) != 0) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);   // racing first calls store the same address
+    }
+    *out = p;
+    return hipSuccess;
 }
 
 enum { kMaskNone = 0, kMaskBlockCausal = 1, kMaskVdnWindow = 2 };
@@ -170,6 +199,8 @@ const char* fv_sdpa_arch(void) { return "gfx950"; }
 int fv_sdpa_init(void) {
     hipError_t e = fv_internal_init_flash();
     if (e == hipSuccess) e = fv_internal_init_vsa();
+    void* p = nullptr;
+    if (e == hipSuccess) e = static_scratch(&p);
     return e == hipSuccess ? FV_OK : fail_hip(e, "fv_sdpa_init");
 }
 
@@ -241,6 +272,42 @@ int fv_sdpa_dense_bf16_splitkv(const uint16_t* q, const uint16_t* k, const uint1
     m.splits = splits ? splits : 1;
     m.workspace = workspace;
     m.workspace_bytes = workspace_bytes;
+    return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, m, stream);
+}
+
+size_t fv_sdpa_splitkv_static_bytes(void) { return kStaticScratchBytes; }
+
+int fv_sdpa_dense_bf16_splitkv_static(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
+                                      int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
+                                      size_t q_rows, size_t k_rows, size_t v_rows, size_t splits, void* stream) {
+    if (!fv_sdpa_supported(1, bh, sq, sk, d)) return decline("sdpa: shape not taken by the fused kernel");
+    if (splits == 0) splits = fv_sdpa_splitkv_choose(bh, sq, sk);
+    // the split count flash_common will settle on (no empty split), to size the partials before launching
+    const size_t nkt = (sk + 63) / 64;
+    if (splits > 1) {
+        const size_t per = (nkt + splits - 1) / splits;
+        splits = (nkt + per - 1) / per;
+    }
+    MaskArgs m;
+    m.q_rows = q_rows;
+    m.k_rows = k_rows;
+    m.v_rows = v_rows;
+    m.splits = splits ? splits : 1;
+    if (m.splits > 1) {
+        const size_t need = fv_sdpa_splitkv_workspace_bytes(bh, sq, d, m.splits);
+        if (need > kStaticScratchBytes) {
+            char buf[200];
+            snprintf(buf, sizeof buf,
+                     "sdpa: split-KV partials of this call need %zu bytes, the static buffer holds %zu "
+                     "(use fv_sdpa_dense_bf16_splitkv with a workspace)", need, kStaticScratchBytes);
+            return fv_invalid(buf);
+        }
+        void* p = nullptr;
+        const hipError_t e = static_scratch(&p);
+        if (e != hipSuccess) return fail_hip(e, "sdpa: resolving the static split-KV buffer");
+        m.workspace = p;
+        m.workspace_bytes = kStaticScratchBytes;
+    }
     return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, m, stream);
 }
 

@@ -36,6 +36,7 @@ const char* fv_sdpa_arch(void);
  * more than 64 KB (`hipFuncSetAttribute`, the reference's `opt_in_dynamic_shared`, rt/ops.rs:1445-1461).
  * Optional: every entry point does this itself at its first launch on a device; call it before
  * capturing a HIP graph whose first launch of a kernel would otherwise fall inside the capture.
+ * Also resolves this device's address of the static split-KV buffer (fv_sdpa_dense_bf16_splitkv_static).
  * Idempotent, thread-safe. */
 int fv_sdpa_init(void);
 
@@ -76,6 +77,22 @@ int fv_sdpa_dense_bf16_splitkv(const uint16_t* q, const uint16_t* k, const uint1
                                int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                                size_t q_rows, size_t k_rows, size_t v_rows, size_t splits, void* workspace,
                                size_t workspace_bytes, void* stream);
+
+/* fv_sdpa_dense_bf16_splitkv for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference. The
+ * partial results live in a buffer inside the library's own code object (a file-scope __device__ array of
+ * fv_sdpa_splitkv_static_bytes() = 32 MiB per GPU, held until the process ends) instead of a caller
+ * workspace, and the call makes no hipMalloc / hipFree of any kind. splits == 0 takes
+ * fv_sdpa_splitkv_choose's count. A shape whose partials need more than the buffer
+ * (fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits) > fv_sdpa_splitkv_static_bytes()) is refused with
+ * -hipErrorInvalidValue and a message; nothing is launched. Every call on a GPU shares that GPU's one
+ * buffer: calls that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered.
+ * Nothing in the buffer has to start at zero (every split writes all of its rows before the merge reads
+ * them). Results are bit-identical to fv_sdpa_dense_bf16_splitkv with the same split count. */
+size_t fv_sdpa_splitkv_static_bytes(void);
+int fv_sdpa_dense_bf16_splitkv_static(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
+                                      int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
+                                      size_t q_rows, size_t k_rows, size_t v_rows, size_t splits, void* stream);
 
 /* rt/attn.rs:652-730 `device_mma_sdpa_causal` + kernels/attn2.cu:626-642
  * `flash_mma_fwd2_causal_d128`: the same under BlockCausal{block_tokens,
