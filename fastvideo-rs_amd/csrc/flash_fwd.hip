@@ -45,9 +45,10 @@
 // matrix phase m in slot 2m and VALU phase m in slot 2m+1; group 1 is one slot
 // behind. K and V tiles rotate through 4 LDS buffers each (128 KB): matrix phase
 // m reads K(2m), K(2m+1), V(2m-2), V(2m-1) and issues K(2m+2), K(2m+3), V(2m),
-// V(2m+1) into the buffers phase m-1 read last, from descriptors (addresses, tail
-// clamp) prepared in the VALU phase before, so the matrix phase carries bare DMA
-// instructions and no branches (a branch inside the unrolled phase breaks the
+// V(2m+1) into the buffers phase m-1 read last, all of them during the first tile
+// of the pair (a load needs more than a thousand cycles to land), from descriptors
+// (addresses, tail clamp) prepared in the VALU phase before, so the matrix phase
+// carries bare DMA instructions and no branches (a branch inside the unrolled phase breaks the
 // register allocation of the 16-register accumulator tuples: 59 spills measured).
 // Every wave waits for its own loads at the end of the same phase, one barrier
 // before phase m+1 of either group reads them. Phase 0 has no previous pair and runs its QK half only
@@ -278,38 +279,37 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         __builtin_amdgcn_s_setprio(1);
         constexpr int kAhead = MASKED ? 2 : 3;
         const int g0 = first ? D / 16 : 0;   // the first phase starts at the K groups
-        // DMA issue slots: after groups 1, 2 (first tile of the pair) and 4, 5 (second) at
-        // D = 128; after groups 1 and 3 at D = 64 (one instruction per tile and wave)
-        auto hook_k = [&](int g) {
+        // DMA issue slots: all of the phase's loads go out during the FIRST tile of the pair, one
+        // instruction after each of its first groups, in the order the next phase reads the tiles
+        // (V of its first tile, K of its first tile, then the second tile's). A load takes well over
+        // a thousand cycles to land when every CU streams K/V; issued from the second tile's groups
+        // they were still in flight at the end of the phase (330 cycles of every matrix phase
+        // spent in the wait below, measured with shader-clock stamps).
+        auto hook_dma = [&](int g) {
             g -= g0;
             if constexpr (kIt == 2) {
-                if (g == 1) Dma::issue_prepared(dk0, 0);
-                if (g == 2) Dma::issue_prepared(dk0, 1);
-                if (g == 4) Dma::issue_prepared(dk1, 0);
-                if (g == 5) Dma::issue_prepared(dk1, 1);
+                if (g == 0) Dma::issue_prepared(dv0, 0);
+                if (g == 1) Dma::issue_prepared(dv0, 1);
+                if (g == 2) Dma::issue_prepared(dk0, 0);
+                if (g == 3) Dma::issue_prepared(dk0, 1);
+                if (g == 4) Dma::issue_prepared(dv1, 0);
+                if (g == 5) Dma::issue_prepared(dv1, 1);
+                if (g == 6) Dma::issue_prepared(dk1, 0);
+                if (g == 7) Dma::issue_prepared(dk1, 1);
             } else {
+                if (g == 0) Dma::issue_prepared(dv0, 0);
                 if (g == 1) Dma::issue_prepared(dk0, 0);
+                if (g == 2) Dma::issue_prepared(dv1, 0);
                 if (g == 3) Dma::issue_prepared(dk1, 0);
             }
         };
-        auto hook_v = [&](int g) {
-            g -= g0;
-            if constexpr (kIt == 2) {
-                if (g == 1) Dma::issue_prepared(dv0, 0);
-                if (g == 2) Dma::issue_prepared(dv0, 1);
-                if (g == 4) Dma::issue_prepared(dv1, 0);
-                if (g == 5) Dma::issue_prepared(dv1, 1);
-            } else {
-                if (g == 1) Dma::issue_prepared(dv0, 0);
-                if (g == 3) Dma::issue_prepared(dv1, 0);
-            }
-        };
+        auto hook_none = [](int) {};
         if (first) {
-            mfma_phase<false, kAhead, decltype(hook_k)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_k);
-            mfma_phase<false, kAhead, decltype(hook_v)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_v);
+            mfma_phase<false, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_dma);
+            mfma_phase<false, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_none);
         } else {
-            mfma_phase<true, kAhead, decltype(hook_k)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_k);
-            mfma_phase<true, kAhead, decltype(hook_v)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_v);
+            mfma_phase<true, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_dma);
+            mfma_phase<true, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_none);
         }
         __builtin_amdgcn_s_setprio(0);
         wait_vmcnt<0>();             // this wave's loads of this phase have landed
