@@ -5,6 +5,7 @@
 
 #include <limits.h>
 #include <math.h>
+#include <stdlib.h>
 
 #include "fv_internal.h"
 
@@ -47,6 +48,17 @@ VsaWorkspace vsa_layout(size_t bh, size_t nb, size_t topk, size_t dim) {
 extern "C" {
 
 // ---- host geometry ------------------------------------------------------------------
+
+double fv_vsa_default_sparsity(void) {
+    const char* v = getenv("FASTVIDEO_VSA_SPARSITY");
+    if (!v) return 0.8;
+    while (*v == ' ' || *v == '\t' || *v == '\n' || *v == '\r') v++;
+    char* end = nullptr;
+    const double x = strtod(v, &end);
+    if (end == v) return 0.8;
+    while (*end == ' ' || *end == '\t' || *end == '\n' || *end == '\r') end++;
+    return *end == '\0' ? x : 0.8;
+}
 
 size_t fv_vsa_topk_for(double sparsity, size_t num_tiles) {
     double keep = ceil((1.0 - sparsity) * (double)num_tiles);

@@ -231,7 +231,8 @@ int kv_rope_bhsd(const void* x, DType x_dtype, size_t x_rows, const float* cos_t
     return e == hipSuccess ? FV_OK : fv_fail_hip(e, "rope_bhsd");
 }
 
-CausalKvCache::CausalKvCache(KvSpec s, size_t num_layers) : spec(s), layers_(num_layers) {}
+CausalKvCache::CausalKvCache(KvSpec s, size_t num_layers, bool static_mode)
+    : spec(s), layers_(num_layers), static_mode_(static_mode) {}
 
 CausalKvCache::~CausalKvCache() {
     for (auto& l : layers_) {
@@ -258,7 +259,8 @@ std::vector<KvPointers> CausalKvCache::pointers() const {
 
 Result<bool> CausalKvCache::set_pointers(const std::vector<KvPointers>& p) {
     std::lock_guard<std::mutex> g(mu_);
-    if (p.size() != layers_.size()) return kv_msg("causal kv: set_pointers needs a static cache and one entry per layer");
+    if (!static_mode_ || p.size() != layers_.size())
+        return kv_msg("causal kv: set_pointers needs a static cache and one entry per layer");
     for (size_t i = 0; i < p.size(); i++) {
         layers_[i].global_end = p[i].global_end;
         layers_[i].local_end = p[i].local_end;
@@ -270,6 +272,7 @@ Result<bool> CausalKvCache::set_pointers(const std::vector<KvPointers>& p) {
 
 Result<bool> CausalKvCache::advance(size_t current_start, size_t n, size_t sink_target) {
     std::lock_guard<std::mutex> g(mu_);
+    if (!static_mode_) return kv_msg("causal kv: advance needs a static cache");
     // plan every layer first, so that an error leaves no layer moved
     std::vector<KvMove> moves;
     for (const Layer& L : layers_) {
@@ -330,6 +333,7 @@ Result<std::pair<Tensor, Tensor>> CausalKvCache::update(size_t layer, const Tens
         skip = spec.sink > mv.local_start ? spec.sink - mv.local_start : 0;
         if (skip > n) skip = n;
     }
+    if (!static_mode_) return update_dynamic(L, mv, skip, k, v, current_start, st);
     if (!L.k) {
         const size_t cap = spec.capacity > n ? spec.capacity : n;
         if (b * h == 0 || cap == 0 || d == 0 || dv == 0) return kv_msg("causal kv: empty keys");
@@ -376,6 +380,72 @@ Result<std::pair<Tensor, Tensor>> CausalKvCache::update(size_t layer, const Tens
     return std::make_pair(std::move(kw), std::move(vw));
 }
 
+// wan/causal.rs:556-624, the `new` (non-static) mode of `update`: the layer's K / V become
+// cat(kept prefix, block) in new buffers of exactly local_end tokens; the roll is part of the copy
+// ([0, sink) and [sink + evicted, prev) land back to back), everything after the block is dropped.
+Result<std::pair<Tensor, Tensor>> CausalKvCache::update_dynamic(Layer& L, const KvMove& mv, size_t skip, const Tensor& k,
+                                                                const Tensor& v, size_t current_start, hipStream_t st) {
+    const size_t b = k.shape[0], h = k.shape[1], n = k.shape[2], d = k.shape[3], dv = v.shape[3], bh = b * h;
+    if (bh == 0 || d == 0 || dv == 0 || mv.local_end == 0) return kv_msg("causal kv: empty keys");
+    if (L.k && (L.b != b || L.h != h || L.d != d || L.dv != dv || L.kd != k.dtype || L.vd != v.dtype))
+        return kv_msg("causal kv: keys [" + std::to_string(b) + ", " + std::to_string(h) + ", .., " + std::to_string(d) +
+                      "] do not continue the cached [" + std::to_string(L.b) + ", " + std::to_string(L.h) + ", .., " +
+                      std::to_string(L.d) + "]");
+    const size_t prev = L.k ? L.local_end : 0, at = mv.local_start + skip, len_new = mv.local_end;
+    // what survives of the old tokens, as (source start, count) pieces laid back to back from 0
+    size_t piece_from[2] = {0, 0}, piece_len[2] = {prev, 0};
+    if (mv.evicted > 0) {
+        const size_t sink = std::min(spec.sink, prev), tail_start = std::min(sink + mv.evicted, prev);
+        piece_len[0] = sink;
+        piece_from[1] = tail_start;
+        piece_len[1] = prev - tail_start;
+    }
+    if (at > piece_len[0] + piece_len[1]) {
+        if (prev == 0) return kv_msg("causal kv: write past an empty cache");
+        return kv_msg("causal kv: write at " + std::to_string(at) + " leaves a gap after " +
+                      std::to_string(piece_len[0] + piece_len[1]) + " cached tokens");
+    }
+    void *nk = nullptr, *nv = nullptr;
+    hipError_t e = hipMallocAsync(&nk, bh * len_new * d * esize(k.dtype), st);
+    if (e == hipSuccess) e = hipMallocAsync(&nv, bh * len_new * dv * esize(v.dtype), st);
+    if (e == hipSuccess && spec.rebase_sink && spec.sink > 0 && !L.raw_sink) e = hipMalloc(&L.raw_sink, bh * spec.sink * d * 4);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        if (nk) (void)hipFreeAsync(nk, st);
+        if (nv) (void)hipFreeAsync(nv, st);
+        return kv_msg(std::string("causal kv: allocating the layer's buffers: ") + hipGetErrorString(e));
+    }
+    int rc = FV_OK;
+    size_t dst = 0;
+    for (int p = 0; p < 2 && rc == FV_OK; p++) {
+        const size_t take = std::min(piece_len[p], at - std::min(at, dst));   // the prefix ends at the write position
+        if (take > 0) {
+            rc = kv_copy_tokens(nk, len_new, dst, L.k, L.cap, piece_from[p], take, bh, d, k.dtype, st);
+            if (rc == FV_OK) rc = kv_copy_tokens(nv, len_new, dst, L.v, L.cap, piece_from[p], take, bh, dv, v.dtype, st);
+        }
+        dst += take;
+    }
+    if (rc == FV_OK && n > skip) {
+        rc = kv_copy_tokens(nk, len_new, at, k.data, n, skip, n - skip, bh, d, k.dtype, st);
+        if (rc == FV_OK) rc = kv_copy_tokens(nv, len_new, at, v.data, n, skip, n - skip, bh, dv, v.dtype, st);
+    }
+    if (rc != FV_OK) {
+        (void)hipFreeAsync(nk, st);
+        (void)hipFreeAsync(nv, st);
+        return kv_msg(std::string("causal kv: write: ") + fv_sdpa_last_error());
+    }
+    if (L.k) (void)hipFreeAsync(L.k, st);   // stream-ordered: the copies above have read them by then
+    if (L.v) (void)hipFreeAsync(L.v, st);
+    L.k = nk, L.v = nv;
+    L.b = b, L.h = h, L.cap = len_new, L.d = d, L.dv = dv, L.kd = k.dtype, L.vd = v.dtype;
+    L.global_end = current_start + n;
+    L.local_end = len_new;
+    const size_t len = len_new - mv.window_start;
+    Tensor kw = Tensor::window((char*)L.k + mv.window_start * d * esize(L.kd), {b, h, len, d}, L.kd, L.cap);
+    Tensor vw = Tensor::window((char*)L.v + mv.window_start * dv * esize(L.vd), {b, h, len, dv}, L.vd, L.cap);
+    return std::make_pair(std::move(kw), std::move(vw));
+}
+
 // wan/causal.rs:739-776 `rebase_sink`, static mode
 Result<bool> CausalKvCache::rebase_sink(size_t target, const float* orig_cos, const float* orig_sin,
                                         const float* new_cos, const float* new_sin, hipStream_t st) {
@@ -408,7 +478,7 @@ Result<bool> CausalKvCache::rebase_sink(size_t target, const float* orig_cos, co
 
 struct fv_kv_cache {
     fv::rt::CausalKvCache cache;
-    fv_kv_cache(fv::rt::KvSpec s, size_t layers) : cache(s, layers) {}
+    fv_kv_cache(fv::rt::KvSpec s, size_t layers, bool static_mode) : cache(s, layers, static_mode) {}
 };
 
 extern "C" {
@@ -440,15 +510,24 @@ int fv_kv_shift_tokens_down(void* t, size_t rows, size_t from, size_t to, size_t
                                         is_bf16 ? fv::rt::DType::Bf16 : fv::rt::DType::F32, (hipStream_t)stream);
 }
 
-fv_kv_cache* fv_kv_cache_new(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
-                             int rope_policy, size_t layers) {
+static fv_kv_cache* kv_cache_make(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
+                                  int rope_policy, size_t layers, bool static_mode) {
     fv::rt::KvSpec s;
     s.capacity = capacity, s.sink = sink, s.max_attention = max_attention, s.frame_tokens = frame_tokens;
     s.rolling = rolling != 0;
     s.relativistic = rope_policy == FV_KV_ROPE_RELATIVISTIC;
     s.rebase_sink = rope_policy == FV_KV_ROPE_REBASED_SINK && sink > 0;
-    return new fv_kv_cache(s, layers);
+    return new fv_kv_cache(s, layers, static_mode);
 }
+fv_kv_cache* fv_kv_cache_new(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
+                             int rope_policy, size_t layers) {
+    return kv_cache_make(capacity, sink, max_attention, frame_tokens, rolling, rope_policy, layers, true);
+}
+fv_kv_cache* fv_kv_cache_new_dynamic(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
+                                     int rope_policy, size_t layers) {
+    return kv_cache_make(capacity, sink, max_attention, frame_tokens, rolling, rope_policy, layers, false);
+}
+int fv_kv_cache_is_static(const fv_kv_cache* c) { return c && c->cache.is_static() ? 1 : 0; }
 
 int fv_rope_bhsd(const void* x, int x_is_bf16, size_t x_rows, const float* cos_t, const float* sin_t, int negate_sin,
                  void* out, int out_is_bf16, size_t out_rows, size_t bh, size_t s, size_t d, void* stream) {

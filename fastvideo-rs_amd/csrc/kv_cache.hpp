@@ -66,10 +66,14 @@ struct KvPointers {
     bool raw_valid = false;
 };
 
-// wan/causal.rs:341-723, `new_static` mode.
+// wan/causal.rs:341-723. static_mode (`new_static`): persistent buffers written in place, the same
+// addresses at every block forward (what a HIP-graph replay needs). Otherwise (`new`): every write
+// builds the layer's K / V anew, exactly local_end tokens long (kept prefix + the block), in freshly
+// allocated stream-ordered buffers, and releases the previous ones; the windows hold the same values.
 class CausalKvCache {
   public:
-    CausalKvCache(KvSpec spec, size_t num_layers);
+    CausalKvCache(KvSpec spec, size_t num_layers, bool static_mode = true);
+    bool is_static() const { return static_mode_; }
     ~CausalKvCache();
     CausalKvCache(const CausalKvCache&) = delete;
     CausalKvCache& operator=(const CausalKvCache&) = delete;
@@ -121,9 +125,12 @@ class CausalKvCache {
         DType kd = DType::F32, vd = DType::F32;
         size_t global_end = 0, local_end = 0;
     };
+    Result<std::pair<Tensor, Tensor>> update_dynamic(Layer& L, const KvMove& mv, size_t skip, const Tensor& k,
+                                                     const Tensor& v, size_t current_start, hipStream_t st);
     mutable std::mutex mu_;
     std::vector<Layer> layers_;
     bool sink_guard_ = false;
+    const bool static_mode_;
 };
 
 }  // namespace fv::rt

@@ -8,7 +8,12 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <stdio.h>
+
 #include <atomic>
+#include <mutex>
+#include <set>
+#include <string>
 #include <tuple>
 
 #include "../../include/fv_sdpa_hip.h"
@@ -136,6 +141,35 @@ bool env_flag(const char* name, bool dflt) {
              strcasecmp(v, "no") == 0);
 }
 
+// rt/log.rs: FASTVIDEO_LOG unset / "1" / "info" = info, "2" / "debug" / "trace" / "verbose" = debug,
+// "0" / "off" / "false" / "quiet" / "error" = quiet (trimmed, case-insensitive); read once.
+int log_level_from(const char* v) {
+    if (!v) return 1;
+    std::string s(v);
+    const size_t a = s.find_first_not_of(" \t\r\n"), b = s.find_last_not_of(" \t\r\n");
+    s = a == std::string::npos ? std::string() : s.substr(a, b - a + 1);
+    for (char& c : s) c = (char)tolower((unsigned char)c);
+    if (s == "0" || s == "off" || s == "false" || s == "quiet" || s == "error") return 0;
+    if (s == "2" || s == "debug" || s == "trace" || s == "verbose") return 2;
+    return 1;
+}
+int log_level() {
+    static const int level = log_level_from(getenv("FASTVIDEO_LOG"));
+    return level;
+}
+
+// One "[fastvideo] sdpa: <kernel> B= H= Sq= Sk= D=" line on stderr the first time a (kernel, shape) pair
+// runs (rt/attn.rs:306-310 logs its fused launches once; a shape is part of the key here so that a
+// run's log shows every attention geometry it used). At most 256 distinct lines per process.
+void log_first_use(const char* kernel, size_t b, size_t h, size_t sq, size_t sk, size_t d) {
+    if (log_level() < 1) return;
+    static std::mutex mu;
+    static std::set<std::tuple<std::string, size_t, size_t, size_t, size_t, size_t>> seen;
+    std::lock_guard<std::mutex> lock(mu);
+    if (seen.size() >= 256 || !seen.emplace(kernel, b, h, sq, sk, d).second) return;
+    fprintf(stderr, "[fastvideo] sdpa: %s B=%zu H=%zu Sq=%zu Sk=%zu D=%zu\n", kernel, b, h, sq, sk, d);
+}
+
 size_t elem_size(DType t) { return t == DType::F32 ? 4 : 2; }
 
 std::string rc_message(int rc) {
@@ -254,6 +288,8 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
     if (rc == FV_DECLINED) return std::optional<Tensor>{};
     if (rc != FV_OK) return TensorError{"sdpa: " + rc_message(rc), rc < 0 ? -rc : 0};
     ((causal || window) ? g_causal : g_fused)++;
+    log_first_use(causal ? "fused mma block-causal" : window ? "fused mma vdn-window" : "fused mma", s->b, s->h, s->sq, s->sk,
+                  s->d);
     return std::optional<Tensor>{std::move(out)};
 }
 
@@ -595,6 +631,7 @@ Result<Tensor> sdpa_composed(const Tensor& q, const Tensor& k, const Tensor& v, 
     if (rc == FV_DECLINED) return msg("sdpa: every kernel of the route declined");
     if (rc != FV_OK) return TensorError{"sdpa: " + rc_message(rc), -rc};
     g_composed++;
+    log_first_use(mask ? "composed f32 (masked)" : "composed f32", b, h, sq, sk, d);
     return std::move(out);
 }
 
@@ -708,6 +745,9 @@ void fv_rt_set_bf16_activations(int v) {
     fv::rt::set_bf16_activations_override(v < 0 ? std::nullopt : std::optional<bool>(v != 0));
 }
 int fv_rt_bf16_activations(void) { return fv::rt::bf16_activations() ? 1 : 0; }
+
+int fv_rt_log_level(void) { return fv::rt::log_level(); }
+int fv_rt_parse_log_level(const char* v) { return fv::rt::log_level_from(v); }
 
 int fv_rt_parse_backend(const char* v) { return (int)fv::rt::parse_backend(v ? v : ""); }
 int fv_rt_backend(void) { return (int)fv::rt::backend(); }

@@ -35,6 +35,8 @@ SIGNATURES = {
     "fv_kv_copy_tokens": (C.c_int, [_vp, _sz, _sz, _vp, _sz, _sz, _sz, _sz, _sz, C.c_int, _vp]),
     "fv_kv_shift_tokens_down": (C.c_int, [_vp, _sz, _sz, _sz, _sz, _sz, _sz, C.c_int, _vp]),
     "fv_kv_cache_new": (_vp, [_sz, _sz, _sz, _sz, C.c_int, C.c_int, _sz]),
+    "fv_kv_cache_new_dynamic": (_vp, [_sz, _sz, _sz, _sz, C.c_int, C.c_int, _sz]),
+    "fv_kv_cache_is_static": (C.c_int, [_vp]),
     "fv_kv_cache_rebase_sink": (C.c_int, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "fv_kv_cache_set_pointers": (C.c_int, [_vp, _vp, _sz]),
     "fv_kv_cache_advance": (C.c_int, [_vp, _sz, _sz, _sz]),
@@ -58,6 +60,9 @@ SIGNATURES = {
     "fv_rt_set_bf16_activations": (None, [C.c_int]),
     "fv_rt_bf16_activations": (C.c_int, []),
     "fv_rt_stats": (None, [_vp]),
+    "fv_rt_log_level": (C.c_int, []),
+    "fv_rt_parse_log_level": (C.c_int, [C.c_char_p]),
+    "fv_vsa_default_sparsity": (C.c_double, []),
     "fv_rt_parse_backend": (C.c_int, [C.c_char_p]),
     "fv_rt_backend": (C.c_int, []),
     "fv_rt_set_backend": (None, [C.c_int]),

@@ -91,12 +91,14 @@ class _DevView:
 
 
 class CausalKvCache:
-    """wan/causal.rs:341-723, static mode: persistent [b, h, capacity, d] buffers per layer."""
+    """wan/causal.rs:341-723. static (`new_static`, the default here): persistent [b, h, capacity, d]
+    buffers per layer, written in place; static=False (`new`): every write builds the layer's K / V anew."""
 
-    def __init__(self, spec, num_layers):
+    def __init__(self, spec, num_layers, static=True):
         self.spec = spec
         self._layers = num_layers
-        self._h = _lib.lib().fv_kv_cache_new(spec.capacity, spec.sink, spec.max_attention, spec.frame_tokens,
+        make = _lib.lib().fv_kv_cache_new if static else _lib.lib().fv_kv_cache_new_dynamic
+        self._h = make(spec.capacity, spec.sink, spec.max_attention, spec.frame_tokens,
                                              int(spec.rolling), spec.rope, num_layers)
         if not self._h:
             raise TensorError("causal kv: could not create the cache")
@@ -130,6 +132,9 @@ class CausalKvCache:
 
     def reset(self):
         _lib.lib().fv_kv_cache_reset(self._h)
+
+    def is_static(self):
+        return bool(_lib.lib().fv_kv_cache_is_static(self._h))
 
     def set_sink_guard(self, on):
         _lib.lib().fv_kv_cache_set_sink_guard(self._h, int(bool(on)))

@@ -52,7 +52,10 @@ class TilePlan:
 class VsaCtx:
     """rt/vsa.rs:326-347: the uploaded tiling and top-k of one latent grid."""
 
-    def __init__(self, grid, sparsity, device="cuda"):
+    def __init__(self, grid, sparsity=None, device="cuda"):
+        if sparsity is None:     # wan/transformer.rs:2194: FASTVIDEO_VSA_SPARSITY, else 0.8
+            sparsity = float(_lib.lib().fv_vsa_default_sparsity())
+        self.sparsity = sparsity
         self.plan = TilePlan(grid)
         self.topk = topk_for(sparsity, self.plan.num_tiles)
         self.seq = self.plan.seq

@@ -178,6 +178,12 @@ int fv_rt_free(void* p, void* stream);
 /* rt/tensor.rs `with_bf16_act`: per-thread override of FASTVIDEO_BF16_ACT; v < 0 clears it. */
 void fv_rt_set_bf16_activations(int v);
 int fv_rt_bf16_activations(void);
+/* rt/log.rs:17-37: the level FASTVIDEO_LOG selects (read once): 0 quiet ("0", "off", "false", "quiet",
+ * "error"), 2 debug ("2", "debug", "trace", "verbose"), 1 info (unset or anything else). At info and above
+ * fv_rt_sdpa writes one "[fastvideo] sdpa: <kernel> B= H= Sq= Sk= D=" line to stderr the first time a
+ * (kernel, shape) pair runs (rt/attn.rs:306-310). fv_rt_parse_log_level parses a value (NULL = unset). */
+int fv_rt_log_level(void);
+int fv_rt_parse_log_level(const char* v);
 /* rt/sdpa_rule.rs:178-219 `Backend`, `parse_backend`, `backend`: FASTVIDEO_SDPA. 0 dense (the
  * default and every unknown value), 1 cublas, 2 flash, 3 host, 4 sparse. fv_rt_set_backend is a
  * per-thread override of the environment (v < 0 clears it). */
@@ -223,6 +229,15 @@ typedef struct fv_kv_cache fv_kv_cache;
 enum { FV_KV_ROPE_ABSOLUTE = 0, FV_KV_ROPE_RELATIVISTIC = 1, FV_KV_ROPE_REBASED_SINK = 2 };
 fv_kv_cache* fv_kv_cache_new(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens, int rolling,
                              int rope_policy, size_t layers);
+/* wan/causal.rs:379-393 `CausalKvCache::new` (not static): every fv_kv_cache_update builds the layer's K / V
+ * anew, exactly local_end tokens long (the tokens kept before the write position, then the block), in
+ * stream-ordered allocations, and releases the previous pair on the same stream; the windows returned hold
+ * the same values as the static cache's (plane_rows = local_end) and are valid until the layer's next
+ * update. Nothing a HIP graph could replay: fv_kv_cache_set_pointers / _advance refuse such a cache. */
+fv_kv_cache* fv_kv_cache_new_dynamic(size_t capacity, size_t sink, size_t max_attention, size_t frame_tokens,
+                                     int rolling, int rope_policy, size_t layers);
+/* wan/causal.rs:395-397 `is_static`. */
+int fv_kv_cache_is_static(const fv_kv_cache* c);
 void fv_kv_cache_free(fv_kv_cache* c);
 void fv_kv_cache_reset(fv_kv_cache* c);
 /* wan/causal.rs:396-418 `set_sink_guard`: a write that re-runs cached frames leaves the sink slots. */
@@ -264,6 +279,11 @@ int fv_kv_cache_update(fv_kv_cache* c, size_t layer, const fv_tensor* k, const f
 
 /* rt/vsa.rs:34-37 `topk_for`: clamp(ceil((1 - sparsity) * num_tiles), 1, max(num_tiles, 1)). Host. */
 size_t fv_vsa_topk_for(double sparsity, size_t num_tiles);
+/* wan/transformer.rs:2194: the sparsity a caller that names none builds its VsaCtx with:
+ * FASTVIDEO_VSA_SPARSITY parsed as f64 (trimmed; unset or unparsable = 0.8). The reference's other VSA
+ * switches (FASTVIDEO_VSA_TOPK, _VSA_KERNEL, _VSA_TMA, _VSA_FUSED, _VSA_GROUP) choose among its kernels or
+ * bound its gather buffer; this library has one kernel per stage and no gather buffer, so they select nothing. */
+double fv_vsa_default_sparsity(void);
 /* rt/vsa.rs:62-109 `TilePlan::new`. Host arrays. dims_out = {tiles_t, tiles_h, tiles_w,
  * seq, padded}; pass NULL arrays to query the dims. Negative return for an empty grid. */
 int fv_vsa_tile_plan(size_t t, size_t h, size_t w, size_t dims_out[5], int32_t* slot_src,

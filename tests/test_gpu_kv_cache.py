@@ -88,18 +88,22 @@ CACHES = [
 ]
 
 
+@pytest.mark.parametrize("static", [True, False])
 @pytest.mark.parametrize("case", CACHES)
 @pytest.mark.parametrize("bf16", [True, False])
-def test_cache_windows_equal_the_oracles(fv, oracle, case, bf16):
+def test_cache_windows_equal_the_oracles(fv, oracle, case, bf16, static):
+    """Static mode (persistent buffers, wan/causal.rs:386-391) and the tensor-per-write mode
+    (wan/causal.rs:379-385, 556-624) return the same windows: the oracle's, bit for bit."""
     import torch
 
     ft, cap_f, sink_f, rolling, blk_f, count = case
-    announce(f"kv cache {case} bf16={bf16}")
+    announce(f"kv cache {case} bf16={bf16} static={static}")
     b, h, d, layers = 2, 3, 64, 2
     n = blk_f * ft
     spec = fv.KvSpec(ft, cap_f * ft, sink_f * ft, cap_f * ft, rolling)
     ospec = oracle.KvSpecO(ft, cap_f * ft, sink_f * ft, cap_f * ft, rolling)
-    cache, ocache = fv.CausalKvCache(spec, layers), oracle.CausalKvCacheO(ospec, layers)
+    cache, ocache = fv.CausalKvCache(spec, layers, static=static), oracle.CausalKvCacheO(ospec, layers)
+    assert cache.is_static() == static
     dt = torch.bfloat16 if bf16 else torch.float32
     rnd = (lambda x: oracle.quantize_bf16(x)) if bf16 else (lambda x: x)
     dev = lambda x: torch.from_numpy(x).cuda().to(dt)  # noqa: E731
@@ -116,7 +120,12 @@ def test_cache_windows_equal_the_oracles(fv, oracle, case, bf16):
                 assert np.array_equal(vw.float().cpu().numpy(), want_v), (layer, i, step)
                 o = ocache.layers[layer]
                 assert cache.pointers(layer) == (o.global_end, o.local_end)
-    assert cache.bytes() == layers * 2 * b * h * max(cap_f * ft, n) * d * (2 if bf16 else 4)
+    if static:
+        assert cache.bytes() == layers * 2 * b * h * max(cap_f * ft, n) * d * (2 if bf16 else 4)
+    else:   # exactly the cached tokens
+        assert cache.bytes() == sum(2 * b * h * cache.pointers(layer)[1] * d * (2 if bf16 else 4) for layer in range(layers))
+        with pytest.raises(fv.TensorError, match="needs a static cache"):
+            cache.advance(0, n)
     # a new rollout keeps the buffers and starts from empty pointers
     cache.reset()
     ocache.reset()
@@ -127,13 +136,14 @@ def test_cache_windows_equal_the_oracles(fv, oracle, case, bf16):
     assert np.array_equal(kw.float().cpu().numpy(), ocache.update(0, rnd(k), rnd(v), 0)[0])
 
 
-def test_update_keeps_prefix_and_window(fv):
+@pytest.mark.parametrize("static", [True, False])
+def test_update_keeps_prefix_and_window(fv, static):
     """The reference's known answers for `update` (causal.rs:1111-1152), each token's value repeated
     over a 4-wide head dim (the device copies move 16-byte units)."""
     import torch
 
-    announce("kv cache known answers")
-    cache = fv.CausalKvCache(fv.KvSpec(2, 8, 2, 8, True), 1)
+    announce(f"kv cache known answers static={static}")
+    cache = fv.CausalKvCache(fv.KvSpec(2, 8, 2, 8, True), 1, static=static)
     blk = lambda base: (base + torch.arange(4, dtype=torch.float32, device="cuda")).reshape(1, 1, 4, 1).repeat(1, 1, 1, 4)  # noqa: E731
 
     def flat(w):
@@ -274,6 +284,32 @@ def test_rope_bhsd_bit_exact(fv, oracle, in16, out16):
         torch.cuda.synchronize()
         assert got.dtype == (torch.bfloat16 if out16 else torch.float32)
         assert np.array_equal(got.float().cpu().numpy(), want)
+
+
+def test_rebased_sink_in_the_tensor_per_write_mode(fv, oracle):
+    """The rebased-sink policy on a cache that is not static: same contents as the oracle's after every roll."""
+    import torch
+
+    announce("kv rebased sink, tensor-per-write mode")
+    b, h, d, ft = 1, 2, 64, 4
+    win_f, sink_f, blk_f = 6, 2, 2
+    n, sink = blk_f * ft, sink_f * ft
+    spec = fv.KvSpec.rolling_window(ft, win_f, sink_f, fv.KvRope.REBASED_SINK)
+    ospec = oracle.KvSpecO(ft, win_f * ft, sink, win_f * ft, True, rebase_sink=True)
+    cache, ocache = fv.CausalKvCache(spec, 1, static=False), oracle.CausalKvCacheO(ospec, 1)
+    dev = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+    cos_o, sin_o = _rope_tables(30, sink, d)
+    for blk in range(6):
+        target = spec.sink_target((blk + 1) * blk_f)
+        if target > 0:
+            cos_n, sin_n = _rope_tables(30, sink, d, frame0=float(target * ft))
+            cache.rebase_sink(target, (dev(cos_o), dev(sin_o)), (dev(cos_n), dev(sin_n)))
+            ocache.rebase_sink(target, (cos_o, sin_o), (cos_n, sin_n), quantize=None)
+        k, v = _blocks(140 + blk, b, h, n, d, 1)[0]
+        want_k, want_v = ocache.update(0, k, v, blk * n)
+        kw, vw = cache.update(0, dev(k), dev(v), blk * n)
+        torch.cuda.synchronize()
+        assert np.array_equal(kw.cpu().numpy(), want_k) and np.array_equal(vw.cpu().numpy(), want_v), blk
 
 
 @pytest.mark.parametrize("bf16", [True, False])

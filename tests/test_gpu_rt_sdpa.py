@@ -255,3 +255,41 @@ def test_allocation_failure_is_reported_with_its_own_code_and_leaves_the_device_
     got = fv.sdpa(buf, buf, buf, fv.Plan.dense(None))
     torch.cuda.synchronize()
     assert got.shape == buf.shape and torch.isfinite(got.float()).all()
+
+
+def test_first_use_of_a_kernel_on_a_shape_is_logged_once():
+    """rt/attn.rs:306-310 + rt/log.rs: at FASTVIDEO_LOG=info the entry names the kernel it launched, once per
+    (kernel, shape); FASTVIDEO_LOG=0 is quiet. Run in child processes (the level is read once per process)."""
+    import os
+    import subprocess
+    import sys
+
+    from util import PKG, ROOT
+
+    announce("rt first-use log lines")
+    code = (
+        "import sys; sys.path[:0] = %r\n"
+        "import torch, fv_sdpa\n"
+        "x = torch.randn((1, 2, 300, 128), device='cuda').to(torch.bfloat16)\n"
+        "y = torch.randn((1, 2, 200, 128), device='cuda').to(torch.bfloat16)\n"
+        "z = torch.randn((1, 2, 40, 48), device='cuda')\n"
+        "for _ in range(3):\n"
+        "    fv_sdpa.sdpa(x, x, x, fv_sdpa.Plan.dense(None))\n"
+        "    fv_sdpa.sdpa(x, y, y, fv_sdpa.Plan.dense(None))\n"
+        "    fv_sdpa.sdpa(x, x, x, fv_sdpa.Plan.block_causal(None, fv_sdpa.BlockCausal(100, 0, 0)))\n"
+        "    fv_sdpa.sdpa(z, z, z, fv_sdpa.Plan.dense(None))\n"
+        "torch.cuda.synchronize()\n" % [ROOT, PKG])
+
+    def run(level):
+        env = dict(os.environ)
+        env["FASTVIDEO_LOG"] = level
+        r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        return [ln for ln in r.stderr.splitlines() if ln.startswith("[fastvideo] sdpa:")]
+
+    lines = run("info")
+    assert lines == ["[fastvideo] sdpa: fused mma B=1 H=2 Sq=300 Sk=300 D=128",
+                     "[fastvideo] sdpa: fused mma B=1 H=2 Sq=300 Sk=200 D=128",
+                     "[fastvideo] sdpa: fused mma block-causal B=1 H=2 Sq=300 Sk=300 D=128",
+                     "[fastvideo] sdpa: composed f32 B=1 H=2 Sq=40 Sk=40 D=48"], lines
+    assert run("0") == []

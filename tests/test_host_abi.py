@@ -204,3 +204,36 @@ def test_rt_sdpa_reports_an_allocation_failure_with_its_own_code():
     kv = _fake_tensor((1, 2, 8, 128), False)
     rc, msg = _rt_call(q0, kv, kv, kind=1, mask=_fake_tensor((0, 8), False))
     assert rc < -1 and msg.startswith("sdpa: device allocation failed: ")
+
+
+def test_log_level_parses_like_the_reference():
+    # rt/log.rs:17-37
+    parse = fv_sdpa.lib().fv_rt_parse_log_level
+    for v, want in [(None, 1), (b"", 1), (b"1", 1), (b"info", 1), (b"anything", 1), (b"0", 0), (b"off", 0), (b" OFF ", 0),
+                    (b"false", 0), (b"quiet", 0), (b"error", 0), (b"2", 2), (b"debug", 2), (b"Trace", 2), (b"verbose\n", 2)]:
+        assert parse(v) == want, v
+
+
+def _in_subprocess(code, env):
+    import subprocess
+    import sys
+
+    e = dict(os.environ)
+    e.update(env)
+    r = subprocess.run([sys.executable, "-c", "import sys; sys.path[:0] = %r; " % [ROOT, os.path.join(ROOT, "fastvideo-rs_amd")]
+                        + code], capture_output=True, text=True, env=e, timeout=120)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return r.stdout.strip()
+
+
+def test_environment_defaults_are_read_by_the_library():
+    code = "import fv_sdpa; l = fv_sdpa.lib(); print(l.fv_rt_log_level(), l.fv_vsa_default_sparsity())"
+    assert _in_subprocess(code, {"FASTVIDEO_LOG": "debug", "FASTVIDEO_VSA_SPARSITY": " 0.875 "}) == "2 0.875"
+    assert _in_subprocess(code, {"FASTVIDEO_LOG": "0", "FASTVIDEO_VSA_SPARSITY": "sparse"}) == "0 0.8"
+    env = {k: v for k, v in os.environ.items() if k not in ("FASTVIDEO_LOG", "FASTVIDEO_VSA_SPARSITY")}
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, "-c", "import sys; sys.path[:0] = %r; " % [ROOT, os.path.join(ROOT, "fastvideo-rs_amd")]
+                        + code], capture_output=True, text=True, env=env, timeout=120)
+    assert r.stdout.strip() == "1 0.8", r.stderr[-500:]
