@@ -587,12 +587,19 @@ extern "C" hipError_t fv_internal_launch_topk(const float* scores, unsigned* out
                                               hipStream_t st) {
     if (n < 1 || n > kTopkMaxN) return hipErrorInvalidValue;
     const dim3 grid((rows + kTopkRowsPerBlock - 1) / kTopkRowsPerBlock), block(64 * kTopkRowsPerBlock);
-    // keys per lane: the smallest of 4, 8, 16, 32, 64 that holds the row
-    if (n <= 256) hipLaunchKernelGGL(vsa_topk_kernel<4>, grid, block, 0, st, scores, out, rows, n, k);
-    else if (n <= 512) hipLaunchKernelGGL(vsa_topk_kernel<8>, grid, block, 0, st, scores, out, rows, n, k);
-    else if (n <= 1024) hipLaunchKernelGGL(vsa_topk_kernel<16>, grid, block, 0, st, scores, out, rows, n, k);
-    else if (n <= 2048) hipLaunchKernelGGL(vsa_topk_kernel<32>, grid, block, 0, st, scores, out, rows, n, k);
-    else hipLaunchKernelGGL(vsa_topk_kernel<64>, grid, block, 0, st, scores, out, rows, n, k);
+    // keys per lane: the smallest instantiated count that holds the row (624 tiles: 10)
+    const int need = (n + 63) / 64;
+#define FV_TOPK(K) hipLaunchKernelGGL(vsa_topk_kernel<K>, grid, block, 0, st, scores, out, rows, n, k)
+    if (need <= 4) FV_TOPK(4);
+    else if (need <= 8) FV_TOPK(8);
+    else if (need <= 10) FV_TOPK(10);
+    else if (need <= 12) FV_TOPK(12);
+    else if (need <= 16) FV_TOPK(16);
+    else if (need <= 24) FV_TOPK(24);
+    else if (need <= 32) FV_TOPK(32);
+    else if (need <= 48) FV_TOPK(48);
+    else FV_TOPK(64);
+#undef FV_TOPK
     return hipGetLastError();
 }
 

@@ -91,7 +91,10 @@ def test_coarse_scores_bit_exact_and_coarse_output(fv, oracle, nb):
 
 @pytest.mark.parametrize("rows,n,k,tied", [(7, 1, 1, False), (13, 97, 7, False), (13, 97, 50, True), (5, 624, 125, False),
                                            (5, 624, 125, True), (3, 4096, 819, True), (4, 512, 64, False),
-                                           (2, 300, 300, True), (2, 10, 16, False), (3, 257, 1, True)])
+                                           (2, 300, 300, True), (2, 10, 16, False), (3, 257, 1, True),
+                                           # one case per keys-per-lane instantiation boundary (256 .. 4096 wide rows)
+                                           (3, 256, 33, True), (3, 700, 140, True), (3, 768, 1, False), (2, 1025, 512, True),
+                                           (2, 1536, 300, False), (2, 2049, 2049, True), (2, 3072, 7, True), (2, 3073, 600, False)])
 def test_topk_bit_exact(fv, oracle, rows, n, k, tied):
     import torch
 
