@@ -169,7 +169,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             char* ob = out_is_bf16 ? (char*)(out_bf16 + ((size_t)bh * sq + q0) * kD)
                                    : (char*)(out_f32 + ((size_t)bh * sq + q0) * kD);
             const u32x4 zero = {0u, 0u, 0u, 0u};
-            for (int u = tid; u < qlen * units; u += 512) *reinterpret_cast<u32x4*>(ob + (size_t)u * 16) = zero;
+            for (int u = tid; u < qlen * units; u += 512) global_store<u32x4>(ob + (size_t)u * 16, zero);
             return;
         }
     }
@@ -355,7 +355,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                         f32x4 r;
 #pragma unroll
                         for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
-                        *reinterpret_cast<f32x4*>(po + 32 * db + 8 * g + 4 * h) = r;
+                        global_store<f32x4>(po + 32 * db + 8 * g + 4 * h, r);
                     }
                 if (h == 0) p.part_lse[prow] = l_tot > 0.f ? st.ms_used + __builtin_log2f(l_tot) : NEG;
             }
@@ -388,7 +388,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             const int rr = i * kRowsPer + lr;
             const u32x4 val = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(
                 my + rr * kRowB + ((lc ^ (rr & (kCh - 1))) << 4));
-            if (wave * 32 + rr < qlen) *reinterpret_cast<u32x4*>(ob + (size_t)rr * kD + lc * 8) = val;
+            if (wave * 32 + rr < qlen) global_store<u32x4>(ob + (size_t)rr * kD + lc * 8, val);
         }
     } else if (row < qlen) {
         const size_t base = ((size_t)bh * sq + q0 + row) * kD;
@@ -402,9 +402,9 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                 for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
                 if (out_is_bf16) {
                     const bf16x4 rb4 = __builtin_convertvector(r, bf16x4);
-                    *reinterpret_cast<bf16x4*>(out_bf16 + base + d0) = rb4;
+                    global_store<bf16x4>(out_bf16 + base + d0, rb4);
                 } else {
-                    *reinterpret_cast<f32x4*>(out_f32 + base + d0) = r;
+                    global_store<f32x4>(out_f32 + base + d0, r);
                 }
             }
     }

@@ -61,6 +61,14 @@ FV_DEV float pair_sum(float x) {
     return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
 }
 
+// A store through a pointer whose address space the compiler no longer knows (a kernel argument that went
+// through an `asm` pin, an address built from one) is emitted as a FLAT store, which also takes an LDS issue
+// slot and counts against the LDS counter. This names the address space.
+template <class T>
+FV_DEV void global_store(void* p, T v) {
+    *(__attribute__((address_space(1))) T*)p = v;
+}
+
 FV_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // f32 -> bf16 bits, round to nearest even, NaN quiet, overflow to inf: the
