@@ -13,6 +13,7 @@ composed|softmax) are for the design notes; the driver's line is the default `se
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -219,7 +220,7 @@ def bench_kvcache(args, fpb=3):
         "ms_per_step_with_window_copies_no_split": round(copied, 4), "ms_per_step_in_place_no_split": round(unsplit, 4),
         "ms_per_step_eager_python_loop": round(eager, 4),
         "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::flash_fwd_pp2<false, 128>"},
+                     "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::flash_fwd_pp2<false, 128, false>"},
     }
     print(json.dumps(rec), flush=True)
 
@@ -408,7 +409,7 @@ def visible_pairs(sq, sk, bt):
     return total
 
 
-def cpu_baseline(h, sq, sk, d, bt, flops_full, q, k, v, budget_s, gpu_out=None):
+def cpu_baseline(h, sq, sk, d, bt, flops_full, q, k, v, budget_s, gpu_out=None, scale=None):
     """Time the oracle's fp32 composed SDPA on a bounded sample of query rows; with `gpu_out` (the
     kernel's output of the timed launches) also compare those rows, all heads, with the oracle's."""
     import numpy as np
@@ -424,7 +425,7 @@ def cpu_baseline(h, sq, sk, d, bt, flops_full, q, k, v, budget_s, gpu_out=None):
     def run(n):
         rows = np.sort(rng.choice(sq, size=min(n, sq), replace=False)).astype(np.int64)
         t0 = time.perf_counter()
-        want = oracle.sdpa_composed_rows(qn, kn, vn, rows, mask_bc=mask, threads=threads)
+        want = oracle.sdpa_composed_rows(qn, kn, vn, rows, scale=scale, mask_bc=mask, threads=threads)
         return time.perf_counter() - t0, rows, want
 
     t_probe, rows, _ = run(min(16, sq))
@@ -455,6 +456,10 @@ def cpu_baseline(h, sq, sk, d, bt, flops_full, q, k, v, budget_s, gpu_out=None):
     }
 
 
+def lib_is_log2_domain(lib, scale):
+    return lib.fv_sdpa_is_log2_domain_scale(scale) == 1
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -467,6 +472,10 @@ def main():
     ap.add_argument("--inputs", default="randn", choices=["randn", "zeros"],
                     help="attention workloads only. zeros: the same launches on all-zero Q/K/V, a power experiment "
                          "(same instruction stream, no bit activity in the operands); never the headline")
+    ap.add_argument("--fold-scale", type=int, default=0,
+                    help="attention workloads only. 1: Q is drawn as bf16(N(0,1) * scale * log2 e) and the call passes "
+                         "scale = ln 2, what a caller that folds the softmax scale into the q RMSNorm weight does; the "
+                         "kernels then run their form without the per-score multiply-add; never the headline")
     ap.add_argument("--copy-calibration-mib", type=int, default=0,
                     help="also launch one plain device copy of this many MiB (known HBM traffic, to scale "
                          "profiler byte counters); not part of the timed region")
@@ -504,7 +513,14 @@ def main():
     h, sq, sk, bt, desc = WORKLOADS[args.workload]
     d = 64 if args.workload.endswith("_d64") else 128
     g = torch.Generator(device=dev).manual_seed(20240)
-    q = torch.randn((h, sq, d), generator=g, device=dev).to(torch.bfloat16)
+    scale = 1.0 / d ** 0.5
+    q = torch.randn((h, sq, d), generator=g, device=dev)
+    if args.fold_scale:
+        q *= scale * 1.4426950408889634
+        scale = float(torch.tensor(math.log(2.0), dtype=torch.float32).item())
+        if not lib_is_log2_domain(fv_sdpa.lib(), scale):
+            raise RuntimeError("scale = ln 2 does not select the log2-domain form")
+    q = q.to(torch.bfloat16)
     k = torch.randn((h, sk, d), generator=g, device=dev).to(torch.bfloat16)
     v = torch.randn((h, sk, d), generator=g, device=dev).to(torch.bfloat16)
     if args.inputs == "zeros":
@@ -512,7 +528,6 @@ def main():
     out = torch.empty((h, sq, d), device=dev, dtype=torch.bfloat16 if args.out_bf16 else torch.float32)
     lib = fv_sdpa.lib()
     stream = torch.cuda.current_stream().cuda_stream
-    scale = 1.0 / d ** 0.5
 
     def step():
         if bt < 0:
@@ -561,7 +576,8 @@ def main():
         traffic_source += " (rocprofv3 --pmc runs of this command; not measured in this run)"
     rec = {
         "metric": "SDPA TFLOP/s + % bf16 MFMA peak, Wan-1.3B 480p self-attn (S=32760,H=12,d=128)"
-        if args.workload == "self" else f"SDPA TFLOP/s ({args.workload})",
+        if args.workload == "self" and not args.fold_scale else
+        f"SDPA TFLOP/s ({args.workload}{', softmax scale folded into Q' if args.fold_scale else ''})",
         "value": round(value, 3),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -572,7 +588,8 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic" if args.inputs == "randn" else "all-zero operands (power experiment, not a benchmark)",
+        "data": ("synthetic" if args.inputs == "randn" else "all-zero operands (power experiment, not a benchmark)") +
+                (" (Q = bf16(N(0,1) * scale * log2 e), call scale ln 2)" if args.fold_scale else ""),
         "config": {"workload": desc, "H": h, "Sq": sq, "Sk": sk, "d": d, "block_tokens": bt,
                    "out": "bf16" if args.out_bf16 else "f32", "flops_per_call": flops,
                    "dense_equivalent_flops": flops_dense_equiv},
@@ -580,7 +597,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": f"fv::flash_fwd_pp2<{'true' if bt else 'false'}, {d}>",
+                     "kernel": f"fv::flash_fwd_pp2<{'true' if bt else 'false'}, {d}, {'true' if args.fold_scale else 'false'}>",
                      "avg_kernel_ms": round(avg_kernel_ms, 4), "median_kernel_ms": round(kern_ms[len(kern_ms) // 2], 4),
                      "min_hbm_bytes": bytes_min,
                      "hbm_frac_at_min_traffic": round(bytes_min / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
@@ -588,7 +605,8 @@ def main():
     if args.cpu_seconds > 0 and bt >= 0:   # the row-sampled oracle takes dense and block-causal masks
         # outside the timed region; the rows the baseline computes double as a parity sample of this run's output
         parity, rec["cpu_baseline"] = cpu_baseline(h, sq, sk, d, bt, flops, q, k, v, args.cpu_seconds,
-                                                   out if args.inputs == "randn" else None)
+                                                   out if args.inputs == "randn" else None,
+                                                   scale if args.fold_scale else None)
         if parity is not None:
             rec["parity"] = parity
     print(json.dumps(rec), flush=True)

@@ -12,6 +12,7 @@
 // on the global side: lane i fetches the chunk that belongs at its position.
 #pragma once
 #include "fv_common.h"
+#include <type_traits>
 
 namespace fv {
 
@@ -323,6 +324,83 @@ FV_DEV void softmax_tile_pair(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxState& st
     }
 }
 
+// softmax_tile_pair for calls whose scores are in the base-2 log domain already (scale * log2(e) == 1: the
+// caller folded the softmax scale into Q, e.g. into the weight of the q RMSNorm that produced it). The matrix
+// phase starts every S block from `negoff` (16 copies of minus the lane's offset) as its C operand, so the
+// scores arrive as s - off and P = 2^(s - off) is one v_exp_f32 per score with no multiply-add in front of
+// it: a fifth of the softmax's VALU work gone. State per lane (= per query): `off` the offset, `r` the running
+// max relative to it (-inf until the query has seen a finite score), `l_acc` the lane's share of the row sum.
+// When some lane's r exceeds kRescaleLog2 (or a query sees its first finite score) every lane moves its offset
+// to its running max: l and O are scaled by 2^-r, this pair's scores lose r, negoff is rewritten (wave-uniform
+// branch, rare). Same policy and same exactness argument as softmax_tile_pair: P and l always share an offset.
+struct SoftmaxOffState {
+    float r, off, l_acc;
+    FV_DEV void init() {
+        r = neg_inf();
+        off = 0.f;
+        l_acc = 0.f;
+    }
+};
+template <int NO = 4>
+FV_DEV void softmax_tile_pair_off(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxOffState& st, f32x16 (&o)[NO],
+                                  f32x16& negoff, bf16x8 (&pb0)[4], bf16x8 (&pb1)[4]) {
+    const float NEG = neg_inf();
+    float mx = s0[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s0[0][i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s0[1][i]);
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s1[b][i]);
+    mx = pair_max(mx);
+    const float r_new = __builtin_fmaxf(st.r, mx);
+    const bool need = (r_new > kRescaleLog2) || (st.r == NEG && r_new != NEG);
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {
+        const float delta = (r_new == NEG) ? 0.f : r_new;
+        const float alpha = (st.r == NEG) ? 0.f : fast_exp2(-delta);
+        st.l_acc *= alpha;
+#pragma unroll
+        for (int db = 0; db < NO; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                s0[b][i] -= delta;   // -inf stays -inf
+                s1[b][i] -= delta;
+            }
+        st.off += delta;
+#pragma unroll
+        for (int i = 0; i < 16; i++) negoff[i] = -st.off;
+        st.r = (r_new == NEG) ? NEG : 0.f;
+    } else {
+        st.r = r_new;
+    }
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            f32x16 e;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                e[i] = fast_exp2(half ? s1[b][i] : s0[b][i]);
+                st.l_acc += e[i];
+            }
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                f32x8 f;
+#pragma unroll
+                for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
+                if (half) pb1[2 * b + t] = __builtin_convertvector(f, bf16x8);
+                else pb0[2 * b + t] = __builtin_convertvector(f, bf16x8);
+            }
+        }
+    }
+}
+
 // O^T (128 d x 32 queries) += V^T P^T.
 template <int D = 128>
 FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 (&o)[D / 32]) {
@@ -345,7 +423,8 @@ FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 
 // One MFMA phase with a deep, explicit LDS prefetch: O^T += V^T P^T of the
 // previous tile (groups 0-7, if DO_PV) followed by S^T = K Q^T of the current
 // one (groups 8-15). A group is 2 operand fragments (8 VGPRs) feeding 2 MFMAs on
-// different accumulators. kAhead (2-3, bounded by the 256-VGPR budget) groups are always in flight ahead of the group
+// different accumulators; the first K MFMA of a key block takes `s_init` as its C operand (zeros, or minus the
+// softmax offset of the lane's query). kAhead (2-3, bounded by the 256-VGPR budget) groups are always in flight ahead of the group
 // being multiplied, so an MFMA waits on a read issued kAhead x 64 cycles of
 // matrix-pipe time earlier instead of on LDS latency plus the 64 B/clk per-SIMD
 // LDS return path. sched_barrier keeps the compiler from re-serialising reads
@@ -353,7 +432,7 @@ FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 
 template <bool DO_PV, int kAhead, class Hook, int D = 128>
 FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& rb,
                        const bf16x8 (&pb)[4], f32x16 (&o)[D / 32], const bf16x8 (&qf)[D / 16],
-                       f32x16 (&s)[2], Hook&& hook) {
+                       f32x16 (&s)[2], const f32x16& s_init, Hook&& hook) {
     using G = TileGeo<D>;
     constexpr int NV = G::kVGroups, NG = G::kGroups;
     constexpr int G0 = DO_PV ? 0 : NV;
@@ -384,11 +463,9 @@ FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& 
                 o[db] = mfma32(f[g][x], pb[t], o[db]);
             }
         } else {
-            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
-                                 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int x = 0; x < 2; x++)   // S is born at dk == 0, not before the PV part
-                s[x] = mfma32(f[g][x], qf[g - NV], g == NV ? zero : s[x]);
+            for (int x = 0; x < 2; x++)   // S is born at dk == 0, not before the PV part, from the C operand s_init
+                s[x] = mfma32(f[g][x], qf[g - NV], g == NV ? s_init : s[x]);
         }
     };
 #pragma unroll

@@ -66,7 +66,10 @@ constexpr int kBN = 64;          // keys per tile
 constexpr int kPpBM = 256;      // queries per workgroup
 constexpr int kRing2 = 4;        // K buffers = V buffers: 128 KB of LDS at D = 128, 64 KB at D = 64
 
-template <bool MASKED, int D>
+// LOG2DOM: the call's scale * log2(e) is exactly 1 (scores are base-2 logarithms as they leave the MFMAs):
+// the softmax offset rides in the C operand of the K Q^T MFMAs and the per-score multiply-add is gone
+// (softmax_tile_pair_off).
+template <bool MASKED, int D, bool LOG2DOM>
 __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     using G = TileGeo<D>;
     constexpr int kD = D;
@@ -218,8 +221,12 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     for (int db = 0; db < kNO; db++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o[db][i] = 0.f;
-    SoftmaxState st;
+    std::conditional_t<LOG2DOM, SoftmaxOffState, SoftmaxState> st;
     st.init();
+    // the C operand every S block starts from: zeros, or (LOG2DOM) minus the lane's softmax offset
+    f32x16 s_init;
+#pragma unroll
+    for (int i = 0; i < 16; i++) s_init[i] = 0.f;
     f32x16 s0[2], s1[2];
     bf16x8 pb0[4], pb1[4];     // P of the previous pair of tiles (first read in phase 1; defined from the start)
 #pragma unroll
@@ -305,11 +312,11 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         };
         auto hook_none = [](int) {};
         if (first) {
-            mfma_phase<false, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_dma);
-            mfma_phase<false, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_none);
+            mfma_phase<false, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, s_init, hook_dma);
+            mfma_phase<false, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, s_init, hook_none);
         } else {
-            mfma_phase<true, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, hook_dma);
-            mfma_phase<true, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, hook_none);
+            mfma_phase<true, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, s_init, hook_dma);
+            mfma_phase<true, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, s_init, hook_none);
         }
         __builtin_amdgcn_s_setprio(0);
         wait_vmcnt<0>();             // this wave's loads of this phase have landed
@@ -319,7 +326,8 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         // ---- VALU phase: group 0 in slot 2m+1, group 1 in slot 2m+2 ----
         mask_tile(s0, 2 * m);
         mask_tile(s1, 2 * m + 1);
-        softmax_tile_pair<kNO>(s0, s1, st, o, sl2, pb0, pb1);
+        if constexpr (LOG2DOM) softmax_tile_pair_off<kNO>(s0, s1, st, o, s_init, pb0, pb1);
+        else softmax_tile_pair<kNO>(s0, s1, st, o, sl2, pb0, pb1);
         // P and the row sum must be complete before the barrier: without this the
         // compiler sinks the exponentials past it, into the matrix phase
         asm volatile("" ::"v"(pb0[0]), "v"(pb0[1]), "v"(pb0[2]), "v"(pb0[3]), "v"(pb1[0]), "v"(pb1[1]),
@@ -357,7 +365,10 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                         for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
                         global_store<f32x4>(po + 32 * db + 8 * g + 4 * h, r);
                     }
-                if (h == 0) p.part_lse[prow] = l_tot > 0.f ? st.ms_used + __builtin_log2f(l_tot) : NEG;
+                float lse_off;
+                if constexpr (LOG2DOM) lse_off = st.off;
+                else lse_off = st.ms_used;
+                if (h == 0) p.part_lse[prow] = l_tot > 0.f ? lse_off + __builtin_log2f(l_tot) : NEG;
             }
             return;
         }
@@ -466,27 +477,37 @@ extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 
 namespace {
 // The kernel's dynamic LDS limit (128 KB at D = 128), once per device.
-template <bool MASKED, int D>
+template <bool MASKED, int D, bool LOG2DOM>
 hipError_t flash_attr() {
     static std::atomic<unsigned long long> attr_done;
     constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
-    return fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<MASKED, D>, lds, attr_done);
+    return fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<MASKED, D, LOG2DOM>, lds, attr_done);
 }
+template <bool MASKED, int D, bool LOG2DOM>
+hipError_t launch_flash_as(const fv::FlashParams* p, hipStream_t stream) {
+    constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
+    hipError_t e = flash_attr<MASKED, D, LOG2DOM>();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((fv::flash_fwd_pp2<MASKED, D, LOG2DOM>), dim3(p->per_xcd * 8), dim3(512), lds, stream, *p);
+    return hipGetLastError();
+}
+// A call whose scale * log2(e) is exactly 1 (scale = ln 2: the caller folded the softmax scale into Q) runs
+// the form without the per-score multiply-add.
 template <bool MASKED, int D>
 hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
-    constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
-    hipError_t e = flash_attr<MASKED, D>();
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((fv::flash_fwd_pp2<MASKED, D>), dim3(p->per_xcd * 8), dim3(512), lds, stream, *p);
-    return hipGetLastError();
+    return p->sl2 == 1.0f ? launch_flash_as<MASKED, D, true>(p, stream) : launch_flash_as<MASKED, D, false>(p, stream);
 }
 }  // namespace
 
 extern "C" hipError_t fv_internal_init_flash(void) {
-    hipError_t e = flash_attr<false, 128>();
-    if (e == hipSuccess) e = flash_attr<true, 128>();
-    if (e == hipSuccess) e = flash_attr<false, 64>();
-    if (e == hipSuccess) e = flash_attr<true, 64>();
+    hipError_t e = flash_attr<false, 128, false>();
+    if (e == hipSuccess) e = flash_attr<true, 128, false>();
+    if (e == hipSuccess) e = flash_attr<false, 64, false>();
+    if (e == hipSuccess) e = flash_attr<true, 64, false>();
+    if (e == hipSuccess) e = flash_attr<false, 128, true>();
+    if (e == hipSuccess) e = flash_attr<true, 128, true>();
+    if (e == hipSuccess) e = flash_attr<false, 64, true>();
+    if (e == hipSuccess) e = flash_attr<true, 64, true>();
     return e;
 }
 

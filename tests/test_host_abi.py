@@ -40,6 +40,23 @@ def test_supported_table():
     assert not ok(0, 8, 1024, 1024, 128) and not ok(2, 40000, 64, 64, 128)
 
 
+def test_log2_domain_scale_predicate():
+    # scale = ln 2 as f32 times the library's f32 log2(e) rounds to exactly one; its neighbours and the
+    # usual 1/sqrt(d) do not
+    is_log2 = fv_sdpa.lib().fv_sdpa_is_log2_domain_scale
+    ln2 = np.float32(np.log(2.0))
+    assert is_log2(float(ln2)) == 1
+    assert is_log2(float(np.nextafter(ln2, np.float32(0)))) == 0 and is_log2(float(np.nextafter(ln2, np.float32(1)))) == 0
+    for d in (64, 128):
+        assert is_log2(1.0 / np.sqrt(d)) == 0
+    header = open(os.path.join(ROOT, "include", "fv_sdpa_hip.h")).read()
+    m = re.search(r"#define FV_SDPA_SCALE_LOG2_DOMAIN ([0-9.]+)f", header)
+    assert m and np.float32(float(m.group(1))) == ln2
+    rust = open(os.path.join(ROOT, "rust", "fastvideo-hip-sdpa", "src", "ffi.rs")).read()
+    m = re.search(r"FV_SDPA_SCALE_LOG2_DOMAIN: f32 = ([0-9._]+);", rust)
+    assert m and np.float32(float(m.group(1).replace("_", ""))) == ln2
+
+
 @pytest.mark.parametrize("grid", [(4, 4, 4), (33, 28, 52), (3, 5, 7), (1, 1, 1), (1, 1, 5), (21, 30, 52), (32, 32, 32)])
 def test_tile_plan_equals_oracle(oracle, grid):
     got, want = fv_sdpa.TilePlan(grid), oracle.TilePlan(grid)
