@@ -70,3 +70,12 @@ def test_other_workloads_emit_one_json_line(workload):
     rec = json.loads(lines[0])
     assert rec["n_gpus"] == 1 and rec["value"] > 0 and "workload" in rec["config"] and "roofline" in rec
     assert rec["roofline"]["bound"] in ("mfma", "hbm") and 0 < rec["roofline"]["frac"] < 1.0
+
+
+@pytest.mark.gpu
+def test_folded_scale_run_is_labelled_and_checks_its_own_output():
+    r = run(["--workload", "tiny", "--fold-scale", "1", "--steps", "2", "--warmup", "1", "--cpu-seconds", "1"])
+    assert r.returncode == 0, r.stderr[-2000:]
+    rec = json.loads([x for x in r.stdout.splitlines() if x.strip()][-1])
+    assert "folded" in rec["metric"] and "ln 2" in rec["data"] and rec["roofline"]["kernel"].endswith("true>")
+    assert rec["parity"]["ok"]
