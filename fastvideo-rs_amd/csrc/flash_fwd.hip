@@ -493,11 +493,16 @@ hipError_t launch_flash_as(const fv::FlashParams* p, hipStream_t stream) {
 }
 // A call whose scale * log2(e) is exactly 1 (scale = ln 2: the caller folded the softmax scale into Q) runs
 // the form without the per-score multiply-add.
+std::atomic<unsigned long long> g_log2_domain_launches{0};
 template <bool MASKED, int D>
 hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
-    return p->sl2 == 1.0f ? launch_flash_as<MASKED, D, true>(p, stream) : launch_flash_as<MASKED, D, false>(p, stream);
+    if (p->sl2 != 1.0f) return launch_flash_as<MASKED, D, false>(p, stream);
+    g_log2_domain_launches.fetch_add(1, std::memory_order_relaxed);
+    return launch_flash_as<MASKED, D, true>(p, stream);
 }
 }  // namespace
+
+extern "C" uint64_t fv_sdpa_log2_domain_launches(void) { return g_log2_domain_launches.load(std::memory_order_relaxed); }
 
 extern "C" hipError_t fv_internal_init_flash(void) {
     hipError_t e = flash_attr<false, 128, false>();

@@ -55,6 +55,8 @@ int fv_sdpa_supported(size_t b, size_t h, size_t sq, size_t sk, size_t d);
  * math at the same operands and scale. fv_sdpa_is_log2_domain_scale: 1 when `scale` selects that form. */
 #define FV_SDPA_SCALE_LOG2_DOMAIN 0.6931471805599453f /* ln 2 */
 int fv_sdpa_is_log2_domain_scale(float scale);
+/* Launches of that form since the library was loaded (all fused entries together). */
+uint64_t fv_sdpa_log2_domain_launches(void);
 
 /* rt/attn.rs:283-421 `device_mma_sdpa_with` + kernels/attn2.cu:607-621
  * `flash_mma_fwd2_d128` / `_d64`: out = softmax(scale * q k^T) v.

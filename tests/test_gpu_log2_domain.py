@@ -37,12 +37,27 @@ def folded_qkv(oracle, seed, bh, sq, sk, d, std=1.0):
     return (q, k, v), (qf, oracle.quantize_bf16(k), oracle.quantize_bf16(v))
 
 
-def test_the_predicate(fv):
+def test_the_predicate_and_the_form_taken(fv, oracle):
+    import torch
+
     lib = fv.lib()
     assert lib.fv_sdpa_is_log2_domain_scale(LN2) == 1
     for d in (64, 128):
         assert lib.fv_sdpa_is_log2_domain_scale(1.0 / math.sqrt(d)) == 0
     assert lib.fv_sdpa_is_log2_domain_scale(1.0) == 0
+    # the launch counter moves with calls at scale ln 2, through every fused entry, and with no other call
+    _, (qf, kr, vr) = folded_qkv(oracle, 5000, 2, 300, 300, 128)
+    qd, kd, vd = (to_dev_bf16(x) for x in (qf, kr, vr))
+    n0 = lib.fv_sdpa_log2_domain_launches()
+    fv.sdpa_dense_bf16(qd, kd, vd)
+    fv.sdpa_block_causal_bf16(qd, kd, vd, 100, 0, 0)
+    assert lib.fv_sdpa_log2_domain_launches() == n0
+    fv.sdpa_dense_bf16(qd, kd, vd, scale=LN2)
+    fv.sdpa_block_causal_bf16(qd, kd, vd, 100, 0, 0, scale=LN2)
+    fv.sdpa_vdn_window_bf16(qd, kd, vd, 10, 20, 14, 0, 1, scale=LN2)
+    fv.sdpa_dense_bf16_splitkv(qd, kd, vd, splits=2, scale=LN2)
+    torch.cuda.synchronize()
+    assert lib.fv_sdpa_log2_domain_launches() == n0 + 4
 
 
 SHAPES = [  # (bh, sq, sk, std, d)

@@ -19,7 +19,7 @@ HEADER = os.path.join(ROOT, "include", "fv_sdpa_hip.h")
 
 # C type (const-ness and pointer depth kept) -> (Rust type, ctypes class or None for void)
 BASE = {"int": ("c_int", C.c_int), "float": ("f32", C.c_float), "double": ("f64", C.c_double),
-        "size_t": ("usize", C.c_size_t), "long long": ("c_longlong", C.c_longlong)}
+        "size_t": ("usize", C.c_size_t), "long long": ("c_longlong", C.c_longlong), "uint64_t": ("u64", C.c_uint64)}
 POINTEE = {"void": "c_void", "char": "c_char", "float": "f32", "uint16_t": "u16", "uint32_t": "u32", "int32_t": "i32",
            "uint64_t": "u64", "size_t": "usize", "int": "c_int", "fv_tensor": "FvTensor", "fv_plan": "FvPlan",
            "fv_kv_cache": "FvKvCache"}
