@@ -102,3 +102,73 @@ def test_seeded_case(fv, oracle, kind, seed):
         got = fv.vsa_topk(torch.from_numpy(s).cuda(), kk)
         torch.cuda.synchronize()
         assert np.array_equal(got.cpu().numpy().view(np.uint32), oracle.topk_device_order(s, kk))
+
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("kind", KINDS[:4])
+def test_seeded_case_log2_domain(fv, oracle, kind, seed):
+    """The same sweep through the form for calls at scale ln 2 (softmax scale folded into Q before its rounding)."""
+    import math
+
+    import torch
+
+    from util import randn
+
+    rng = np.random.Generator(np.random.PCG64(50000 + 1000 * KINDS.index(kind) + seed))
+    d = int(rng.choice([64, 128]))
+    bh = int(rng.integers(1, 5))
+    sq, sk = int(rng.integers(1, 700)), int(rng.integers(1, 900))
+    data_seed = int(rng.integers(0, 1 << 30))
+    ln2 = float(np.float32(math.log(2.0)))
+    assert fv.lib().fv_sdpa_is_log2_domain_scale(ln2) == 1
+
+    def operands(nq, nk):
+        sl2 = np.float32(1.0 / math.sqrt(d)) * np.float32(1.4426950408889634)
+        q = oracle.quantize_bf16(randn(data_seed, (bh, nq, d)) * sl2)
+        return q, oracle.quantize_bf16(randn(data_seed + 1, (bh, nk, d))), oracle.quantize_bf16(randn(data_seed + 2, (bh, nk, d)))
+
+    if kind == "dense":
+        announce(f"sweep log2 dense bh={bh} sq={sq} sk={sk} d={d} seed={data_seed}")
+        q, k, v = operands(sq, sk)
+        got = fv.sdpa_dense_bf16(*(to_dev_bf16(x) for x in (q, k, v)), scale=ln2)
+        torch.cuda.synchronize()
+        assert_parity(got.cpu().numpy(), oracle.sdpa_composed(q, k, v, scale=ln2), f"sweep_log2_dense_{seed}")
+    elif kind == "block_causal":
+        if seed % 2:
+            sk = sq
+        bt = int(rng.integers(1, max(2, max(sq, sk))))
+        win, sink = int(rng.integers(0, 4)), int(rng.integers(0, 3))
+        announce(f"sweep log2 causal bh={bh} sq={sq} sk={sk} d={d} block={bt} window={win} sink={sink} seed={data_seed}")
+        q, k, v = operands(sq, sk)
+        out = torch.full((bh, sq, d), float("nan"), device="cuda")
+        fv.sdpa_block_causal_bf16(*(to_dev_bf16(x) for x in (q, k, v)), bt, win, sink, scale=ln2, out=out)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        tq, tk = np.arange(sq)[:, None] // bt, np.arange(sk)[None, :] // bt
+        live = ((tk < sink) | ((tk <= tq) & ((win == 0) | (tq - tk < win)))).any(axis=1)
+        assert np.isfinite(got).all() and np.all(got[:, ~live] == 0.0)
+        if live.any():
+            want = oracle.sdpa_f64(q, k, v, scale=ln2, mask_bc=(bt, win, sink), rows=np.nonzero(live)[0])
+            assert_parity(got[:, live], want, f"sweep_log2_causal_{seed}")
+    elif kind == "vdn_window":
+        ft, frames = int(rng.integers(1, 60)), int(rng.integers(1, 12))
+        vs, tail = int(rng.integers(0, 50)), int(rng.integers(0, 50))
+        s = vs + ft * frames + tail
+        chunk, radius = int(rng.integers(0, 4)), int(rng.integers(0, 4))
+        announce(f"sweep log2 vdn bh={bh} s={s} d={d} start={vs} ft={ft} frames={frames} chunk={chunk} radius={radius} seed={data_seed}")
+        q, k, v = operands(s, s)
+        got = fv.sdpa_vdn_window_bf16(*(to_dev_bf16(x) for x in (q, k, v)), vs, ft, frames, chunk, radius, scale=ln2)
+        torch.cuda.synchronize()
+        mask = oracle.vdn_window_dense_mask(vs, ft, frames, chunk, radius, s, s)
+        assert_parity(got.cpu().numpy(), oracle.sdpa_composed(q, k, v, scale=ln2, mask=mask), f"sweep_log2_vdn_{seed}")
+    else:
+        sk2 = sk + 600
+        off, splits = int(rng.integers(0, 77)), int(rng.integers(1, 9))
+        announce(f"sweep log2 splitkv bh={bh} sq={sq} sk={sk2} d={d} offset={off} splits={splits} seed={data_seed}")
+        q, k, v = operands(sq, sk2 + 77)
+        tk, tv = to_dev_bf16(k), to_dev_bf16(v)
+        got = fv.sdpa_dense_bf16_splitkv(to_dev_bf16(q), tk[:, off:off + sk2], tv[:, off:off + sk2], splits=splits, scale=ln2)
+        torch.cuda.synchronize()
+        want = oracle.sdpa_composed(q, np.ascontiguousarray(k[:, off:off + sk2]), np.ascontiguousarray(v[:, off:off + sk2]),
+                                    scale=ln2)
+        assert_parity(got.cpu().numpy(), want, f"sweep_log2_splitkv_{seed}")
