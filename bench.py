@@ -125,7 +125,7 @@ def bench_vsa(args):
         "whole_op_tile_ordered_inputs_ms": {"avg": round(avg_t, 4), "median": round(med_t, 4), "wall": round(wall_t, 4)},
         "stages_median_ms": {k2: round(v2, 4) for k2, v2 in stages.items()},
         "roofline": {"bound": "mfma", "achieved": round(fine_tflops, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(fine_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::vsa_fine_kernel",
+                     "frac": round(fine_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::vsa_fine_kernel<false>",
                      "avg_kernel_ms": round(stages["fine"], 4),
                      "banded_selection_tflops": round(flops / (stages["fine_banded_selection"] * 1e-3) / 1e12, 3)},
     }

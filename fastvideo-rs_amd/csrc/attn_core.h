@@ -189,17 +189,17 @@ FV_DEV void qk_tile(const lds_u8* kb, int k_base, const bf16x8 (&qf)[8], f32x16 
     }
 }
 
-// qk_tile with `side(g)` after MFMA g (0..15): side work that rides under the matrix pipe.
+// qk_tile with `side(g)` after MFMA g (0..15): side work that rides under the matrix pipe. Every S block
+// starts from `s_init` (the C operand of its first MFMA): zeros, or minus the softmax offset of the lane's query.
 template <class Side>
-FV_DEV void qk_tile_side(const lds_u8* kb, int k_base, const bf16x8 (&qf)[8], f32x16 (&s)[2], Side&& side) {
+FV_DEV void qk_tile_side(const lds_u8* kb, int k_base, const bf16x8 (&qf)[8], f32x16 (&s)[2], const f32x16& s_init,
+                         Side&& side) {
 #pragma unroll
     for (int b = 0; b < 2; b++) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) s[b][i] = 0.f;
-#pragma unroll
         for (int dk = 0; dk < 8; dk++) {
             const bf16x8 a = lds_read_b128(kb + (k_base ^ (dk << 5)) + b * 32 * kRowBytes);
-            s[b] = mfma32(a, qf[dk], s[b]);
+            s[b] = mfma32(a, qf[dk], dk == 0 ? s_init : s[b]);
             __builtin_amdgcn_sched_barrier(0);
             side(b * 8 + dk);
             __builtin_amdgcn_sched_barrier(0);
@@ -398,6 +398,59 @@ FV_DEV void softmax_tile_pair_off(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxOffSt
                 else pb0[2 * b + t] = __builtin_convertvector(f, bf16x8);
             }
         }
+    }
+}
+
+// softmax_tile_side for scores in the base-2 log domain (see softmax_tile_pair_off): one tile, with the side slots
+// of softmax_tile_side.
+template <class Side>
+FV_DEV void softmax_tile_side_off(f32x16 (&s)[2], SoftmaxOffState& st, f32x16 (&o)[4], f32x16& negoff,
+                                  bf16x8 (&pb)[4], Side&& side) {
+    const float NEG = neg_inf();
+    float mx = s[0][0];
+#pragma unroll
+    for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s[0][i]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s[1][i]);
+    mx = pair_max(mx);
+    const float r_new = __builtin_fmaxf(st.r, mx);
+    const bool need = (r_new > kRescaleLog2) || (st.r == NEG && r_new != NEG);
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {
+        const float delta = (r_new == NEG) ? 0.f : r_new;
+        const float alpha = (st.r == NEG) ? 0.f : fast_exp2(-delta);
+        st.l_acc *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) s[b][i] -= delta;   // -inf stays -inf
+        st.off += delta;
+#pragma unroll
+        for (int i = 0; i < 16; i++) negoff[i] = -st.off;
+        st.r = (r_new == NEG) ? NEG : 0.f;
+    } else {
+        st.r = r_new;
+    }
+    side(0);
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+        f32x16 e;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            e[i] = fast_exp2(s[b][i]);
+            st.l_acc += e[i];
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            f32x8 f;
+#pragma unroll
+            for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
+            pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
+        }
+        side(1 + b);
     }
 }
 

@@ -331,6 +331,9 @@ __global__ __launch_bounds__(256) void vsa_tile_qkv3_kernel(Three t, const int* 
 // by direct global->LDS loads: K(i+1) streams in under softmax/PV of tile i and
 // V(i) under QK/softmax of tile i. 32 KB of LDS per workgroup, so four
 // workgroups share a CU.
+// LOG2DOM: the call's scale * log2(e) is exactly 1 (the caller folded the softmax scale into Q): the softmax offset
+// rides in the C operand of the K Q^T MFMAs and the per-score multiply-add is gone (softmax_tile_side_off).
+template <bool LOG2DOM>
 __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     lds_u8* kbuf = (lds_u8*)smem_raw;
@@ -360,8 +363,11 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
     for (int db = 0; db < 4; db++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o[db][i] = 0.f;
-    SoftmaxState st;
+    std::conditional_t<LOG2DOM, SoftmaxOffState, SoftmaxState> st;
     st.init();
+    f32x16 s_init;   // the C operand every S block starts from: zeros, or (LOG2DOM) minus the lane's softmax offset
+#pragma unroll
+    for (int i = 0; i < 16; i++) s_init[i] = 0.f;
 
     // Per-lane DMA offsets are loop-invariant (every tile has 64 rows in the tile-ordered layout), so a
     // tile load is 8 (m0, load) pairs from a scalar base. The tile indices and sizes of the next two
@@ -382,7 +388,7 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
         // in three groups through the softmax: issued in one burst they hold the wave (in-order issue)
         // while the CU's address path drains, 4 % of the kernel's time
         const uint16_t* vsrc = vb + (size_t)tile * kTileElems * 128;
-        qk_tile_side(kbuf, rb.k, qf, s, [&](int g) {
+        qk_tile_side(kbuf, rb.k, qf, s, s_init, [&](int g) {
             if (g & 1) dma.template issue_one<true>(vbuf, vsrc, wave, g >> 1);
         });
         block_barrier();     // K buffer free
@@ -398,13 +404,15 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
                 }
         }
         bf16x8 pb[4];
-        softmax_tile_side(s, st, o, sl2, pb, [&](int part) {
+        auto k_loads = [&](int part) {
             if (more) {
                 const int first = 3 * part, last = part == 2 ? 8 : first + 3;
 #pragma unroll
                 for (int it = first; it < last; it++) dma.template issue_one<false>(kbuf, ksrc, wave, it);
             }
-        });
+        };
+        if constexpr (LOG2DOM) softmax_tile_side_off(s, st, o, s_init, pb, k_loads);
+        else softmax_tile_side(s, st, o, sl2, pb, k_loads);
         if (more) wait_vmcnt<8>(); else wait_vmcnt<0>();   // V(i) landed; K(i+1) may be in flight
         block_barrier();
         pv_tile(vbuf, rb.v, pb, o);
@@ -618,7 +626,10 @@ extern "C" hipError_t fv_internal_launch_tile_qkv(const void* x, int x_is_bf16, 
 }
 
 extern "C" hipError_t fv_internal_launch_fine(const fv::VsaFineParams* p, hipStream_t st) {
-    hipLaunchKernelGGL(vsa_fine_kernel, dim3(p->per_xcd * 8), dim3(128), 2 * kTileBytes, st, *p);
+    if (p->sl2 == 1.0f)   // scale = ln 2: the caller folded the softmax scale into Q
+        hipLaunchKernelGGL(vsa_fine_kernel<true>, dim3(p->per_xcd * 8), dim3(128), 2 * kTileBytes, st, *p);
+    else
+        hipLaunchKernelGGL(vsa_fine_kernel<false>, dim3(p->per_xcd * 8), dim3(128), 2 * kTileBytes, st, *p);
     return hipGetLastError();
 }
 

@@ -351,3 +351,45 @@ def test_full_size_rows_of_ones(fv, grid, sparsity):
     e0, e1 = (out0 - 1.0).abs().max().item(), (out1 - 2.0).abs().max().item()
     print(f"max |out - 1| = {e0:.3e} (zero gate), max |out - 2| = {e1:.3e} (gate of one)")
     assert e0 <= 4e-3 and e1 <= 4e-3
+
+
+@pytest.mark.parametrize("grid", GRIDS)
+def test_log2_domain_form_of_the_fine_stage_and_the_whole_op(fv, oracle, grid):
+    """Calls at scale ln 2 (softmax scale folded into Q before its rounding) run the fine kernel's form without the
+    per-score multiply-add: same bars against the f64 block-sparse attention and the host oracle at the same
+    operands and scale; the block lists stay the host oracle's."""
+    import math
+
+    import torch
+
+    ln2 = float(np.float32(math.log(2.0)))
+    assert fv.lib().fv_sdpa_is_log2_domain_scale(ln2) == 1
+    announce(f"vsa log2-domain grid={grid}")
+    ctx = fv.VsaCtx(grid, 0.8)
+    plan, nb = ctx.plan, ctx.num_tiles
+    oplan = oracle.TilePlan(grid)
+    sl2 = np.float32(1.0 / np.sqrt(D)) * np.float32(1.4426950408889634)
+    bh = 2
+    q = oracle.quantize_bf16(randn(71, (bh, ctx.seq, D)) * sl2)
+    k, v = (oracle.quantize_bf16(randn(71 + i, (bh, ctx.seq, D))) for i in (1, 2))
+    g = oracle.quantize_bf16(randn(74, (bh, ctx.seq, D), 0.5))
+    # fine stage alone, distinct lists
+    topk = max(1, min(nb, 5))
+    sel = np.array([[[(i + h * 7 + j) % nb for j in range(topk)] for i in range(nb)] for h in range(bh)], dtype=np.int32)
+    qt, kt, vt = (fv.vsa_tile_qkv(dev(x), ctx) for x in (q, k, v))
+    sparse = fv.vsa_fine(qt, kt, vt, dev(sel), ctx, ln2)
+    torch.cuda.synchronize()
+    sparse = sparse.cpu().numpy()
+    want = brute_block_sparse(q, k, v, sel, plan, ln2)
+    real = plan.slot_src >= 0
+    got_tok = np.zeros_like(want)
+    got_tok[:, plan.slot_src[real]] = sparse[:, real]
+    assert_parity(got_tok, want, f"vsa_fine_log2_{grid}")
+    # whole op
+    want, want_sel = oracle.vsa_attention_host(q, k, v, g, oplan, ctx.topk, 1, bh, D, np.float32(ln2), return_selected=True)
+    got, sel = fv.vsa_attention_device(dev(q), dev(k), dev(v), dev(g), ctx, ln2, return_selected=True)
+    torch.cuda.synchronize()
+    got, sel = got.cpu().numpy(), sel.cpu().numpy().view(np.uint32)
+    assert np.array_equal(np.sort(sel, -1), np.sort(want_sel.reshape(sel.shape), -1))
+    m = assert_parity(got, want, f"vsa_op_log2_{grid}")
+    assert m["rel_l2"] <= 2e-2
