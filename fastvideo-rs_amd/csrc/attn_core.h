@@ -482,8 +482,11 @@ FV_DEV void pv_tile(const lds_u8* vb, int v_base, const bf16x8 (&pb)[4], f32x16 
 // matrix-pipe time earlier instead of on LDS latency plus the 64 B/clk per-SIMD
 // LDS return path. sched_barrier keeps the compiler from re-serialising reads
 // behind MFMAs.
+// The operand fragments are addressed through per-lane LDS pointers that already hold the buffer's place
+// (`va[db]`: V^T fragments of d block db, `ka[dk]`: K fragments of d chunk dk, both for the FIRST tile of a pair;
+// `tile_off` = 0 or one tile adds the second one as an immediate), so a read costs no address arithmetic.
 template <bool DO_PV, int kAhead, class Hook, int D = 128>
-FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& rb,
+FV_DEV void mfma_phase(const lds_u8* const (&va)[D / 32], const lds_u8* const (&ka)[D / 16], const int tile_off,
                        const bf16x8 (&pb)[4], f32x16 (&o)[D / 32], const bf16x8 (&qf)[D / 16],
                        f32x16 (&s)[2], const f32x16& s_init, Hook&& hook) {
     using G = TileGeo<D>;
@@ -496,16 +499,16 @@ FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& 
 #pragma unroll
             for (int x = 0; x < 2; x++) {
                 const int t = g / kPerT, db = 2 * (g % kPerT) + x;
-                const int a0 = (rb.v ^ (db << 6)) + (16 * t) * G::kRow;
+                const lds_u8* a0 = va[db] + ((16 * t) * G::kRow + tile_off);
                 s16x8 a;
-                a.lo = lds_read_tr16_b64(vb + a0);
-                a.hi = lds_read_tr16_b64(vb + a0 + 8 * G::kRow);
+                a.lo = lds_read_tr16_b64(a0);
+                a.hi = lds_read_tr16_b64(a0 + 8 * G::kRow);
                 f[g][x] = __builtin_bit_cast(bf16x8, a);
             }
         } else {              // K fragments: d chunk dk = g - NV, key blocks 0 and 1
 #pragma unroll
             for (int x = 0; x < 2; x++)
-                f[g][x] = lds_read_b128(kb + (rb.k ^ ((g - NV) << 5)) + x * 32 * G::kRow);
+                f[g][x] = lds_read_b128(ka[g - NV] + (x * 32 * G::kRow + tile_off));
         }
     };
     auto run = [&](int g) {
@@ -531,6 +534,21 @@ FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& 
         __builtin_amdgcn_sched_barrier(0);
         hook(g);   // side work (tile DMA issue) that rides under the matrix pipe
     }
+}
+
+// mfma_phase for one tile given by its V and K buffers (wave-uniform) and the lane's read bases: the fragment
+// addresses are formed here, an add per fragment.
+template <bool DO_PV, int kAhead, class Hook, int D = 128>
+FV_DEV void mfma_phase(const lds_u8* vb, const lds_u8* kb, const TileReadBases& rb,
+                       const bf16x8 (&pb)[4], f32x16 (&o)[D / 32], const bf16x8 (&qf)[D / 16],
+                       f32x16 (&s)[2], const f32x16& s_init, Hook&& hook) {
+    const lds_u8* va[D / 32];
+    const lds_u8* ka[D / 16];
+#pragma unroll
+    for (int db = 0; db < D / 32; db++) va[db] = vb + (rb.v ^ (db << 6));
+#pragma unroll
+    for (int dk = 0; dk < D / 16; dk++) ka[dk] = kb + (rb.k ^ (dk << 5));
+    mfma_phase<DO_PV, kAhead, Hook, D>(va, ka, 0, pb, o, qf, s, s_init, static_cast<Hook&&>(hook));
 }
 
 // Q^T fragments for the wave's 32 queries: rows row0 + lane%32 of a row-major

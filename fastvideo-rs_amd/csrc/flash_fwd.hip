@@ -238,6 +238,19 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         }
 
     typename Dma::Prepared dk0 = target_k(2), dk1 = target_k(3), dv0 = target_v(0), dv1 = target_v(1);
+    // Per-lane LDS addresses of the operand fragments of the first tile of the pair a matrix phase reads: K tiles
+    // 2m, 2m+1 sit in buffers 2 (m & 1) + {0, 1}, V tiles 2m-2, 2m-1 in buffers 2 (1 - m & 1) + {0, 1}, so every
+    // phase flips one bit (two tiles' worth) in each register instead of adding a buffer base to every read.
+    const lds_u8* ka[D / 16];
+    const lds_u8* va[D / 32];
+#pragma unroll
+    for (int dk = 0; dk < D / 16; dk++) ka[dk] = smem + (rb.k ^ (dk << 5));
+#pragma unroll
+    for (int db = 0; db < D / 32; db++) va[db] = smem + ((rb.v ^ (db << 6)) + (kRing2 + 2) * kTileBytes);
+    // (the ring starts at LDS address 0 and spans a power of two, so flipping an address bit moves between buffers)
+    auto flip = [](const lds_u8* q, unsigned bit) -> const lds_u8* {
+        return (const lds_u8*)(__attribute__((address_space(3))) void*)(size_t)((unsigned)(size_t)q ^ bit);
+    };
 
     block_barrier();                 // K(0), K(1) resident
     if (grp == 1) block_barrier();   // group 1 idles through slot 0
@@ -311,12 +324,22 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             }
         };
         auto hook_none = [](int) {};
-        if (first) {
-            mfma_phase<false, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, s_init, hook_dma);
-            mfma_phase<false, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, s_init, hook_none);
+        // (dense launches address the fragments through the flipped pointers; on masked launches, whose phases
+        // read ahead less, that measured 0.6 % slower than an add per fragment, so they keep the adds)
+        if constexpr (MASKED) {
+            if (first) {
+                mfma_phase<false, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, s_init, hook_dma);
+                mfma_phase<false, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, s_init, hook_none);
+            } else {
+                mfma_phase<true, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, s_init, hook_dma);
+                mfma_phase<true, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, s_init, hook_none);
+            }
+        } else if (first) {
+            mfma_phase<false, kAhead, decltype(hook_dma)&, D>(va, ka, 0, pb0, o, qf, s0, s_init, hook_dma);
+            mfma_phase<false, kAhead, decltype(hook_none)&, D>(va, ka, kTileBytes, pb1, o, qf, s1, s_init, hook_none);
         } else {
-            mfma_phase<true, kAhead, decltype(hook_dma)&, D>(vbuf(2 * m - 2), kbuf(2 * m), rb, pb0, o, qf, s0, s_init, hook_dma);
-            mfma_phase<true, kAhead, decltype(hook_none)&, D>(vbuf(2 * m - 1), kbuf(2 * m + 1), rb, pb1, o, qf, s1, s_init, hook_none);
+            mfma_phase<true, kAhead, decltype(hook_dma)&, D>(va, ka, 0, pb0, o, qf, s0, s_init, hook_dma);
+            mfma_phase<true, kAhead, decltype(hook_none)&, D>(va, ka, kTileBytes, pb1, o, qf, s1, s_init, hook_none);
         }
         __builtin_amdgcn_s_setprio(0);
         wait_vmcnt<0>();             // this wave's loads of this phase have landed
@@ -332,6 +355,12 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         // compiler sinks the exponentials past it, into the matrix phase
         asm volatile("" ::"v"(pb0[0]), "v"(pb0[1]), "v"(pb0[2]), "v"(pb0[3]), "v"(pb1[0]), "v"(pb1[1]),
                      "v"(pb1[2]), "v"(pb1[3]), "v"(st.l_acc));
+        if constexpr (!MASKED) {
+#pragma unroll
+            for (int dk = 0; dk < D / 16; dk++) ka[dk] = flip(ka[dk], 2 * kTileBytes);   // the other pair of K buffers
+#pragma unroll
+            for (int db = 0; db < D / 32; db++) va[db] = flip(va[db], 2 * kTileBytes);   // ... and of V buffers
+        }
         dk0 = target_k(2 * m + 4);   // for matrix phase m+1
         dk1 = target_k(2 * m + 5);
         dv0 = target_v(2 * m + 2);
