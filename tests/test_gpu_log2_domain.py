@@ -218,3 +218,39 @@ def test_headline_shape_sampled_rows(fv, oracle):
     want = oracle.sdpa_composed_rows(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), rows,
                                      scale=LN2)
     assert_parity(got.float().cpu().numpy()[:, rows, :], want, "log2_headline_rows")
+
+
+def test_fold_through_the_q_norm_weight(fv, oracle):
+    """The caller's recipe end to end: the q RMSNorm weight carries scale * log2 e, the producer's bf16 kernel
+    rounds q once as it always does, and the SDPA call passes scale = ln 2. The result meets the bars against
+    the oracle on the producer's own output at ln 2, and sits within the fused bar of the unfolded chain
+    (weight w, default scale), whose q differs by the rounding noise of one bf16 product."""
+    import torch
+
+    batch, seq, heads, d = 1, 700, 4, 128
+    announce("fold through q norm weight: prep -> sdpa(ln 2), 1x700x4x128")
+    rng = np.random.Generator(np.random.PCG64(5900))
+    qkv = oracle.quantize_bf16(rng.standard_normal((batch, seq, 3 * heads * d)).astype(np.float32))
+    w = (1.0 + 0.2 * rng.standard_normal(heads * d)).astype(np.float32)
+    theta = rng.uniform(-3.0, 3.0, (seq, d // 2))
+    cos = np.repeat(np.cos(theta), 2, axis=1).astype(np.float32)
+    sin = np.repeat(np.sin(theta), 2, axis=1).astype(np.float32)
+    sl2 = np.float32(1.0 / math.sqrt(d)) * np.float32(1.4426950408889634)
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    x = dev(qkv).to(torch.bfloat16)
+    rope = (dev(cos), dev(sin))
+    k = fv.qk_norm_rope_bhsd(x, heads * d, heads, dev(w), rope).reshape(heads, seq, d)
+    v = fv.split_heads_bhsd(x, 2 * heads * d, heads, d).reshape(heads, seq, d)
+    q_plain = fv.qk_norm_rope_bhsd(x, 0, heads, dev(w), rope).reshape(heads, seq, d)
+    q_fold = fv.qk_norm_rope_bhsd(x, 0, heads, dev(w * sl2), rope).reshape(heads, seq, d)
+    n0 = fv.lib().fv_sdpa_log2_domain_launches()
+    plain = fv.sdpa_dense_bf16(q_plain, k, v)
+    assert fv.lib().fv_sdpa_log2_domain_launches() == n0
+    got = fv.sdpa_dense_bf16(q_fold, k, v, scale=LN2)
+    torch.cuda.synchronize()
+    assert fv.lib().fv_sdpa_log2_domain_launches() == n0 + 1
+    npy = lambda t: t.float().cpu().numpy()  # noqa: E731
+    want = oracle.sdpa_composed(npy(q_fold), npy(k), npy(v), scale=LN2)
+    assert_parity(npy(got), want, "log2_fold_norm_weight")
+    m = metrics(npy(got), npy(plain))
+    assert m["max_abs"] <= 1e-2 and m["cosine"] >= 0.9999, m
