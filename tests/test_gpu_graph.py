@@ -31,10 +31,12 @@ def _fill(g, *tensors):
         t.copy_(torch.randn(t.shape, generator=g, device="cuda").to(t.dtype))
 
 
-def test_dense_and_block_causal_replay(fv):
+@pytest.mark.parametrize("form", ["exact", "log2_domain"])
+def test_dense_and_block_causal_replay(fv, form):
+    """Both forms of the fused kernel (the second is taken at scale = ln 2, operands as they are)."""
     import torch
 
-    announce("graph: dense + block-causal")
+    announce(f"graph: dense + block-causal, {form}")
     bh, s, d = 4, 700, 128
     g = torch.Generator(device="cuda").manual_seed(1)
     q, k, v = (torch.empty((bh, s, d), device="cuda", dtype=torch.bfloat16) for _ in range(3))
@@ -42,7 +44,8 @@ def test_dense_and_block_causal_replay(fv):
     lib = fv.lib()
     out_d = torch.empty((bh, s, d), device="cuda", dtype=torch.bfloat16)
     out_c = torch.empty((bh, s, d), device="cuda", dtype=torch.float32)
-    scale = 1.0 / d ** 0.5
+    scale = 1.0 / d ** 0.5 if form == "exact" else float(np.float32(np.log(2.0)))
+    assert lib.fv_sdpa_is_log2_domain_scale(scale) == (form == "log2_domain")
 
     def run():
         st = torch.cuda.current_stream().cuda_stream
@@ -57,8 +60,8 @@ def test_dense_and_block_causal_replay(fv):
         run()
     for i in range(4):
         _fill(g, q, k, v)
-        want_d = fv.sdpa_dense_bf16(q, k, v, out_bf16=True)
-        want_c = fv.sdpa_block_causal_bf16(q, k, v, 100, 2, 1)
+        want_d = fv.sdpa_dense_bf16(q, k, v, out_bf16=True, scale=scale)
+        want_c = fv.sdpa_block_causal_bf16(q, k, v, 100, 2, 1, scale=scale)
         torch.cuda.synchronize()
         out_d.zero_()
         out_c.zero_()
