@@ -311,8 +311,9 @@ int fv_vsa_tile_mean(const void* x, int x_is_bf16, const int32_t* slot_src, cons
                      float* out, size_t bh, size_t seq, size_t dim, size_t num_tiles, int round16,
                      void* stream);
 /* rt/vsa.rs:385-394 (cuBLAS f32 + kernels/core.cu:177-252 `softmax_last` there):
- * scores[bh, qt, kt] = (qc . kc, summed over d ascending in f32, mul then add) * scale (kept
- * raw: they drive the selection); coarse[bh, qt, :] = softmax(scores[bh, qt, :]) vc.
+ * scores[bh, qt, kt] = the host oracle's arithmetic (rt/vsa.rs:185-189): qc . kc accumulated in f64 over d
+ * ascending, times scale in f64, one rounding to f32 (kept raw: they drive the selection, so the selected
+ * sets equal `vsa_attention_host`'s); coarse[bh, qt, :] = softmax(scores[bh, qt, :]) vc.
  * coarse may be NULL (scores only). num_tiles <= 4096; coarse needs dim == 128. */
 int fv_vsa_coarse(const float* qc, const float* kc, const float* vc, float* scores, float* coarse,
                   size_t bh, size_t num_tiles, size_t dim, float scale, void* stream);
