@@ -52,10 +52,12 @@ int fv_sdpa_supported(size_t b, size_t h, size_t sq, size_t sk, size_t d);
  * fused entry (dense, strided, split-KV, block-causal, VDN window) then runs a form whose softmax offset rides
  * in the C operand of the K Q^T MFMAs and whose multiply-add per score is gone: 3.6 % faster at H=12 S=32760,
  * 8 % on block-causal launches and at head dim 64. Same arithmetic otherwise, same tolerance against the host
- * math at the same operands and scale. fv_sdpa_is_log2_domain_scale: 1 when `scale` selects that form. */
+ * math at the same operands and scale. fv_vsa_fine (and through it fv_vsa_attention, whose coarse stage uses
+ * the scale as given) takes the same form at that scale. fv_sdpa_is_log2_domain_scale: 1 when `scale` selects
+ * that form. */
 #define FV_SDPA_SCALE_LOG2_DOMAIN 0.6931471805599453f /* ln 2 */
 int fv_sdpa_is_log2_domain_scale(float scale);
-/* Launches of that form since the library was loaded (all fused entries together). */
+/* Launches of that form of the dense / masked kernel since the library was loaded (all its entries together). */
 uint64_t fv_sdpa_log2_domain_launches(void);
 
 /* rt/attn.rs:283-421 `device_mma_sdpa_with` + kernels/attn2.cu:607-621
