@@ -246,6 +246,50 @@ def test_full_size_rows_of_ones(fv, bh, s):
     assert err <= 4e-3     # P is rounded to bf16 (2^-9 relative) before it meets V; l sums the unrounded P
 
 
+@pytest.mark.parametrize("form", ["exact", "log2_domain"])
+def test_full_size_permutation_symmetries(fv, form):
+    """Whole-output checks at H = 12, S = 32760 that need no oracle: attention is invariant under a permutation
+    of the keys (applied to K and V alike) and equivariant under a permutation of the queries. A key, a tile or a
+    row indexed wrongly anywhere in the 12 x 32760 x 128 output breaks one of them. The permuted runs visit keys in
+    another order and share rescale decisions with other rows, so the results agree to rounding, not bit for bit:
+    P is rounded to bf16 (2^-9 relative) against offsets that differ between the runs. The bar is set against the
+    output's own scale: max|delta| <= a quarter of the output's standard deviation (and <= 1e-2). The rounding noise
+    measures 0.02 - 0.07 standard deviations at its largest element; one misplaced key tile or row moves its elements
+    by a standard deviation and more."""
+    import torch
+
+    bh, s, d = 12, 32760, 128
+    announce(f"dense headline permutation symmetries, {form}")
+    g = torch.Generator(device="cuda").manual_seed(77)
+    q, k, v = (torch.randn((bh, s, d), generator=g, device="cuda") for _ in range(3))
+    scale = None
+    if form == "log2_domain":
+        q = q * (1.4426950408889634 / d ** 0.5)
+        scale = float(np.float32(np.log(2.0)))
+    q, k, v = (x.to(torch.bfloat16) for x in (q, k, v))
+    base = fv.sdpa_dense_bf16(q, k, v, scale=scale)
+    pk = torch.randperm(s, generator=g, device="cuda")
+    pq = torch.randperm(s, generator=g, device="cuda")
+    by_keys = fv.sdpa_dense_bf16(q, k[:, pk].contiguous(), v[:, pk].contiguous(), scale=scale)
+    by_rows = fv.sdpa_dense_bf16(q[:, pq].contiguous(), k, v, scale=scale)
+    torch.cuda.synchronize()
+    assert torch.isfinite(base).all()
+    dk = (by_keys - base).abs().max().item()
+    dq = (by_rows - base[:, pq]).abs().max().item()
+    bar = min(1e-2, 0.25 * base.std().item())
+    print(f"  key permutation max|delta| {dk:.3e}, query permutation {dq:.3e}, std(out) {base.std().item():.3e}")
+    assert dk <= bar and dq <= bar, (dk, dq, bar)
+    # and the same with a short key axis (cross-attention: 8 key tiles, one of them partial)
+    kc, vc = k[:, :500].contiguous(), v[:, :500].contiguous()
+    pc = torch.randperm(500, generator=g, device="cuda")
+    basec = fv.sdpa_dense_bf16(q, kc, vc, scale=scale)
+    dkc = (fv.sdpa_dense_bf16(q, kc[:, pc].contiguous(), vc[:, pc].contiguous(), scale=scale) - basec).abs().max().item()
+    dqc = (fv.sdpa_dense_bf16(q[:, pq].contiguous(), kc, vc, scale=scale) - basec[:, pq]).abs().max().item()
+    barc = min(1e-2, 0.25 * basec.std().item())
+    print(f"  500 keys: key permutation max|delta| {dkc:.3e}, query permutation {dqc:.3e}, std(out) {basec.std().item():.3e}")
+    assert dkc <= barc and dqc <= barc, (dkc, dqc, barc)
+
+
 @pytest.mark.parametrize("d", [128, 64])
 def test_extreme_score_ranges(fv, oracle, d):
     """Nearly one-hot rows (scores of magnitude ~10^2: the running max jumps by far more than the lazy
