@@ -177,3 +177,32 @@ def test_full_size_masked_rows_of_ones(fv, mode):
     err = (out - 1.0).abs().max().item()
     print(f"max |out - 1| = {err:.3e}")
     assert err <= 4e-3
+
+
+@pytest.mark.parametrize("bt,win,sink", [(1560, 0, 0), (4680, 0, 0), (1560, 4, 1)])
+def test_full_size_prefix_and_block_properties(fv, bt, win, sink):
+    """Whole-output checks at H = 12, S = 21 x 1560 that need no oracle. (1) A block-causal row sees nothing after
+    its own block, so the first n blocks of the full call equal the call on the first n blocks alone, every row
+    and element, bit for bit: the walks visit the same key tiles in the same order, and the keys past the prefix
+    are masked in one call and absent in the other. (2) Without window and sink, the rows of the first block equal
+    dense attention over that block (bar: a quarter of the output's standard deviation, and 1e-2)."""
+    import torch
+
+    bh, frames, ft, d = 12, 21, 1560, 128
+    s = frames * ft
+    announce(f"block-causal full size prefix property bt={bt} win={win} sink={sink}")
+    g = torch.Generator(device="cuda").manual_seed(4242)
+    q, k, v = (torch.randn((bh, s, d), generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    full = fv.sdpa_block_causal_bf16(q, k, v, bt, win, sink)
+    torch.cuda.synchronize()
+    assert torch.isfinite(full).all()
+    for blocks in (1, 2, (s // bt) // 2 + 1):
+        n = blocks * bt
+        part = fv.sdpa_block_causal_bf16(q[:, :n].contiguous(), k[:, :n].contiguous(), v[:, :n].contiguous(), bt, win, sink)
+        torch.cuda.synchronize()
+        assert torch.equal(part, full[:, :n]), (blocks, (part - full[:, :n]).abs().max().item())
+    if win == 0 and sink == 0:
+        first = fv.sdpa_dense_bf16(q[:, :bt].contiguous(), k[:, :bt].contiguous(), v[:, :bt].contiguous())
+        torch.cuda.synchronize()
+        delta = (first - full[:, :bt]).abs().max().item()
+        assert delta <= min(1e-2, 0.25 * first.std().item()), delta
