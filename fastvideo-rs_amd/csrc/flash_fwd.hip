@@ -209,11 +209,32 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         }
     }
     bf16x8 qf[D / 16];
-    {
-        const int row = wave * 32 + c32;
-        load_q_frags<D>(Qh, row, row < qlen, lane, qf);   // drains vmcnt: K(0), K(1) have landed too
-    }
     const TileReadBases rb = tile_read_bases<D>(lane);
+    {
+        // The wave's 32 query rows come through LDS: whole rows by LDS-DMA (1 KB of consecutive global memory per
+        // instruction) into the wave's own slice of the V ring, idle until the first matrix phase requests V(0),
+        // in the K tiles' swizzle, then the fragments with the K operand's conflict-free read pattern. (Loading the
+        // fragments straight from global memory takes 16-byte pieces of 32 rows per instruction: 2 - 3 % slower on
+        // 512-key launches, whose prologue shows; bit-identical.)
+        lds_u8* qs = smem + kRing2 * kTileBytes + wave * (32 * G::kRow);
+        const unsigned qlds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)qs);
+        constexpr int kQIt = 32 * G::kRow / 1024;
+#pragma unroll
+        for (int it = 0; it < kQIt; it++) {
+            const int r = it * G::kRowsPerDma + lane / G::kChunks, pch = lane % G::kChunks;
+            const int rg = min(wave * 32 + r, qlen - 1);   // rows past the end re-read the last one (zeroed below)
+            lds_dma16_s(qlds + it * 1024, Qh, (unsigned)(rg * G::kRow + ((pch ^ G::kswz(r)) << 4)));
+        }
+        wait_vmcnt<0>();   // this wave's rows (and its parts of K(0), K(1)) have landed
+        const bool ok = wave * 32 + c32 < qlen;
+#pragma unroll
+        for (int dk = 0; dk < D / 16; dk++) {
+            bf16x8 t = lds_read_b128(qs + (rb.k ^ (dk << 5)));
+            if (!ok) t = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+            qf[dk] = t;
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the slice is read before any wave passes the barrier below
+    }
 
     constexpr int kNO = D / 32;   // 32-wide d blocks of the accumulator
     f32x16 o[kNO];
