@@ -210,13 +210,15 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     }
     bf16x8 qf[D / 16];
     const TileReadBases rb = tile_read_bases<D>(lane);
-    {
-        // The wave's 32 query rows come through LDS: whole rows by LDS-DMA (1 KB of consecutive global memory per
-        // instruction) into the wave's own slice of the V ring, idle until the first matrix phase requests V(0),
-        // in the K tiles' swizzle, then the fragments with the K operand's conflict-free read pattern. (Loading the
-        // fragments straight from global memory takes 16-byte pieces of 32 rows per instruction: 2 - 3 % slower on
-        // 512-key launches, whose prologue shows; bit-identical.)
-        lds_u8* qs = smem + kRing2 * kTileBytes + wave * (32 * G::kRow);
+    // The wave's 32 query rows come through LDS: whole rows by LDS-DMA (1 KB of consecutive global memory per
+    // instruction) into the wave's own slice of the V ring (group 0: buffers 0, 1, idle until the first matrix
+    // phase requests V(0); group 1: buffers 2, 3, idle a phase longer), in the K tiles' swizzle, then the fragments
+    // with the K operand's conflict-free read pattern. (Loading the fragments straight from global memory takes
+    // 16-byte pieces of 32 rows per instruction: 2 - 3 % slower on 512-key launches, whose prologue shows.)
+    // Group 1, which idles through the first slot anyway, waits for its rows only then: group 0 starts as soon as
+    // K(0), K(1) and its own rows are there.
+    lds_u8* qs = smem + kRing2 * kTileBytes + wave * (32 * G::kRow);
+    auto q_request = [&]() {
         const unsigned qlds = __builtin_amdgcn_readfirstlane((unsigned)(size_t)qs);
         constexpr int kQIt = 32 * G::kRow / 1024;
 #pragma unroll
@@ -225,6 +227,8 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             const int rg = min(wave * 32 + r, qlen - 1);   // rows past the end re-read the last one (zeroed below)
             lds_dma16_s(qlds + it * 1024, Qh, (unsigned)(rg * G::kRow + ((pch ^ G::kswz(r)) << 4)));
         }
+    };
+    auto q_read = [&]() {
         wait_vmcnt<0>();   // this wave's rows (and its parts of K(0), K(1)) have landed
         const bool ok = wave * 32 + c32 < qlen;
 #pragma unroll
@@ -233,7 +237,14 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
             if (!ok) t = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
             qf[dk] = t;
         }
-        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the slice is read before any wave passes the barrier below
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the slice is read before the wave passes its next barrier
+    };
+    if (grp == 0) {
+        q_request();
+        q_read();
+    } else {
+        q_request();
+        wait_vmcnt<32 * G::kRow / 1024>();   // this wave's parts of K(0), K(1); its query rows are still in flight
     }
 
     constexpr int kNO = D / 32;   // 32-wide d blocks of the accumulator
@@ -274,7 +285,10 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     };
 
     block_barrier();                 // K(0), K(1) resident
-    if (grp == 1) block_barrier();   // group 1 idles through slot 0
+    if (grp == 1) {                  // group 1 takes its query rows in slot 0, in which it has nothing else to do
+        q_read();
+        block_barrier();
+    }
 
     // scores of walk position e: keys past the end (or a position past the walk) to -inf;
     // masked launches: keys this lane's query may not see to -inf, skipped when the whole
