@@ -82,6 +82,15 @@ hipError_t static_scratch(void** out) {
 
 enum { kMaskNone = 0, kMaskBlockCausal = 1, kMaskVdnWindow = 2 };
 
+// The split count a launch settles on for `nkt` key tiles when `splits` are asked for: never more splits
+// than key tiles (also keeps the sums below from wrapping on absurd counts), and no empty split.
+size_t settle_splits(size_t nkt, size_t splits) {
+    if (splits <= 1 || nkt <= 1) return 1;
+    if (splits > nkt) splits = nkt;
+    const size_t per = (nkt + splits - 1) / splits;
+    return (nkt + per - 1) / per;
+}
+
 struct MaskArgs {
     int mode = kMaskNone;
     size_t q_rows = 0, k_rows = 0, v_rows = 0;   // rows per (batch, head) plane; 0 = contiguous (sq / sk)
@@ -162,22 +171,18 @@ int flash_common(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* 
     p.part_o = nullptr;
     p.part_lse = nullptr;
     const size_t nkt = (sk + 63) / 64;
-    size_t splits = mode == kMaskNone ? m.splits : 1;
+    size_t splits = mode == kMaskNone ? settle_splits(nkt, m.splits) : 1;
     if (splits > 1) {
-        const size_t per = (nkt + splits - 1) / splits;
-        splits = (nkt + per - 1) / per;             // no empty split
-        if (splits > 1) {
-            if (total * splits > (size_t)INT_MAX / 2) return decline("sdpa: too many workgroups for one launch");
-            const size_t need = fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits);
-            if (!m.workspace || m.workspace_bytes < need || (((uintptr_t)m.workspace) & 255) != 0)
-                return fv_invalid("sdpa: split-KV needs a 256-byte aligned workspace of fv_sdpa_splitkv_workspace_bytes");
-            p.kv_split = (int)splits;
-            p.split_tiles = (int)per;
-            p.part_o = (float*)m.workspace;
-            p.part_lse = (float*)((char*)m.workspace + ((splits * bh * sq * d * 4 + 255) & ~(size_t)255));
-            p.total = (int)(total * splits);
-            p.per_xcd = (p.total + 7) / 8;
-        }
+        if (total * splits > (size_t)INT_MAX / 2) return decline("sdpa: too many workgroups for one launch");
+        const size_t need = fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits);
+        if (!m.workspace || m.workspace_bytes < need || (((uintptr_t)m.workspace) & 255) != 0)
+            return fv_invalid("sdpa: split-KV needs a 256-byte aligned workspace of fv_sdpa_splitkv_workspace_bytes");
+        p.kv_split = (int)splits;
+        p.split_tiles = (int)((nkt + splits - 1) / splits);
+        p.part_o = (float*)m.workspace;
+        p.part_lse = (float*)((char*)m.workspace + ((splits * bh * sq * d * 4 + 255) & ~(size_t)255));
+        p.total = (int)(total * splits);
+        p.per_xcd = (p.total + 7) / 8;
     }
     hipError_t e = fv_internal_launch_flash(&p, mode != kMaskNone ? 1 : 0, (int)d, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip(e, mode != kMaskNone ? "flash_fwd_pp2<masked>" : "flash_fwd_pp2<dense>");
@@ -280,31 +285,39 @@ int fv_sdpa_dense_bf16_splitkv(const uint16_t* q, const uint16_t* k, const uint1
 
 size_t fv_sdpa_splitkv_static_bytes(void) { return kStaticScratchBytes; }
 
+size_t fv_sdpa_splitkv_static_splits(size_t bh, size_t sq, size_t sk, size_t d, size_t splits) {
+    const size_t nkt = (sk + 63) / 64;
+    if (splits != 0) {   // the caller's count, settled as the launch would; refused when its partials do not fit
+        splits = settle_splits(nkt, splits);
+        return fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits) <= kStaticScratchBytes ? splits : 0;
+    }
+    // the library's own choice never refuses: it steps down to the largest count whose partials fit (1 = unsplit)
+    for (size_t s = fv_sdpa_splitkv_choose(bh, sq, sk); s > 1; s--) {
+        const size_t real = settle_splits(nkt, s);
+        if (fv_sdpa_splitkv_workspace_bytes(bh, sq, d, real) <= kStaticScratchBytes) return real;
+    }
+    return 1;
+}
+
 int fv_sdpa_dense_bf16_splitkv_static(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                                       int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                                       size_t q_rows, size_t k_rows, size_t v_rows, size_t splits, void* stream) {
     if (!fv_sdpa_supported(1, bh, sq, sk, d)) return decline("sdpa: shape not taken by the fused kernel");
-    if (splits == 0) splits = fv_sdpa_splitkv_choose(bh, sq, sk);
-    // the split count flash_common will settle on (no empty split), to size the partials before launching
-    const size_t nkt = (sk + 63) / 64;
-    if (splits > 1) {
-        const size_t per = (nkt + splits - 1) / splits;
-        splits = (nkt + per - 1) / per;
+    const size_t run = fv_sdpa_splitkv_static_splits(bh, sq, sk, d, splits);
+    if (run == 0) {
+        char buf[200];
+        snprintf(buf, sizeof buf,
+                 "sdpa: split-KV partials of this call need %zu bytes, the static buffer holds %zu "
+                 "(use fv_sdpa_dense_bf16_splitkv with a workspace)",
+                 fv_sdpa_splitkv_workspace_bytes(bh, sq, d, settle_splits((sk + 63) / 64, splits)), kStaticScratchBytes);
+        return fv_invalid(buf);
     }
     MaskArgs m;
     m.q_rows = q_rows;
     m.k_rows = k_rows;
     m.v_rows = v_rows;
-    m.splits = splits ? splits : 1;
-    if (m.splits > 1) {
-        const size_t need = fv_sdpa_splitkv_workspace_bytes(bh, sq, d, m.splits);
-        if (need > kStaticScratchBytes) {
-            char buf[200];
-            snprintf(buf, sizeof buf,
-                     "sdpa: split-KV partials of this call need %zu bytes, the static buffer holds %zu "
-                     "(use fv_sdpa_dense_bf16_splitkv with a workspace)", need, kStaticScratchBytes);
-            return fv_invalid(buf);
-        }
+    m.splits = run;
+    if (run > 1) {
         void* p = nullptr;
         const hipError_t e = static_scratch(&p);
         if (e != hipSuccess) return fail_hip(e, "sdpa: resolving the static split-KV buffer");

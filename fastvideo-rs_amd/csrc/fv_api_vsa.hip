@@ -49,14 +49,19 @@ extern "C" {
 
 // ---- host geometry ------------------------------------------------------------------
 
+// rt/envflag.rs:32-34 -> settings/parse.rs:43-45: the trimmed value through Rust's `str::parse::<f64>`, 0.8 when
+// unset or unparsable. strtod takes two forms Rust's grammar does not (hex floats, "nan(...)"): refused here, so
+// both sides fall back to the default on the same strings.
 double fv_vsa_default_sparsity(void) {
     const char* v = getenv("FASTVIDEO_VSA_SPARSITY");
     if (!v) return 0.8;
-    while (*v == ' ' || *v == '\t' || *v == '\n' || *v == '\r') v++;
+    while (*v == ' ' || *v == '\t' || *v == '\n' || *v == '\r' || *v == '\v' || *v == '\f') v++;
+    for (const char* c = v; *c; c++)
+        if (*c == 'x' || *c == 'X' || *c == 'p' || *c == 'P' || *c == '(') return 0.8;
     char* end = nullptr;
     const double x = strtod(v, &end);
     if (end == v) return 0.8;
-    while (*end == ' ' || *end == '\t' || *end == '\n' || *end == '\r') end++;
+    while (*end == ' ' || *end == '\t' || *end == '\n' || *end == '\r' || *end == '\v' || *end == '\f') end++;
     return *end == '\0' ? x : 0.8;
 }
 

@@ -31,6 +31,7 @@ SIGNATURES = {
     "fv_sdpa_dense_bf16_splitkv": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float, _sz, _sz, _sz,
                                              _sz, _vp, _sz, _vp]),
     "fv_sdpa_splitkv_static_bytes": (_sz, []),
+    "fv_sdpa_splitkv_static_splits": (_sz, [_sz, _sz, _sz, _sz, _sz]),
     "fv_sdpa_dense_bf16_splitkv_static": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float, _sz, _sz,
                                                     _sz, _sz, _vp]),
     "fv_kv_plan": (C.c_int, [_sz, _sz, _sz, _sz, C.c_int, _sz, _sz, _sz, _sz, _vp]),

@@ -83,7 +83,7 @@ int fv_sdpa_dense_bf16_strided(const uint16_t* q, const uint16_t* k, const uint1
  * them into `out`. Same operands as fv_sdpa_dense_bf16_strided. No counterpart in the reference, whose
  * kernels run one CTA per query tile (rt/attn.rs:378-395). fv_sdpa_splitkv_choose: the split count this
  * library would pick for a shape on the current device (1 = none: use the plain entry; fv_rt_sdpa
- * applies it by itself); splits is clamped so that no split is empty. workspace: 256-byte aligned,
+ * applies it by itself); splits is clamped to the number of 64-key tiles and so that no split is empty. workspace: 256-byte aligned,
  * fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits) bytes. Results agree with the unsplit kernel
  * to rounding (each split normalises by its own row sum before the merge). */
 size_t fv_sdpa_splitkv_choose(size_t bh, size_t sq, size_t sk);
@@ -98,13 +98,17 @@ int fv_sdpa_dense_bf16_splitkv(const uint16_t* q, const uint16_t* k, const uint1
  * partial results live in a buffer inside the library's own code object (a file-scope __device__ array of
  * fv_sdpa_splitkv_static_bytes() = 32 MiB per GPU, held until the process ends) instead of a caller
  * workspace, and the call makes no hipMalloc / hipFree of any kind. splits == 0 takes
- * fv_sdpa_splitkv_choose's count. A shape whose partials need more than the buffer
- * (fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits) > fv_sdpa_splitkv_static_bytes()) is refused with
- * -hipErrorInvalidValue and a message; nothing is launched. Every call on a GPU shares that GPU's one
+ * fv_sdpa_splitkv_choose's count, stepped down to the largest count whose partials fit the buffer (down to
+ * 1 = unsplit), so the library's own choice is never refused. An explicit count whose partials need more
+ * than the buffer (fv_sdpa_splitkv_workspace_bytes(bh, sq, d, splits) > fv_sdpa_splitkv_static_bytes()) is
+ * refused with -hipErrorInvalidValue and a message; nothing is launched.
+ * fv_sdpa_splitkv_static_splits (host arithmetic only): the split count a call with these arguments runs
+ * with (>= 1), or 0 when it would be refused. Every call on a GPU shares that GPU's one
  * buffer: calls that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered.
  * Nothing in the buffer has to start at zero (every split writes all of its rows before the merge reads
  * them). Results are bit-identical to fv_sdpa_dense_bf16_splitkv with the same split count. */
 size_t fv_sdpa_splitkv_static_bytes(void);
+size_t fv_sdpa_splitkv_static_splits(size_t bh, size_t sq, size_t sk, size_t d, size_t splits);
 int fv_sdpa_dense_bf16_splitkv_static(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                                       int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                                       size_t q_rows, size_t k_rows, size_t v_rows, size_t splits, void* stream);

@@ -33,12 +33,22 @@ use std::ptr;
 use ffi::{FvPlan, FvTensor, FV_DECLINED, FV_OK};
 use hip::HipStream;
 
-/// `rt/tensor.rs:92-98`.
-#[derive(Debug, thiserror::Error)]
+/// `rt/tensor.rs:92-98`. `Display` prints the message as it is, which is what the reference's
+/// `#[error("{0}")]` derives; written out by hand so that the crate has no dependency to fetch.
+#[derive(Debug)]
 pub enum TensorError {
-    #[error("{0}")]
     Message(String),
 }
+
+impl std::fmt::Display for TensorError {
+    fn fmt(&self, f: &mut std::fmt::Formatter<'_>) -> std::fmt::Result {
+        match self {
+            TensorError::Message(m) => f.write_str(m),
+        }
+    }
+}
+
+impl std::error::Error for TensorError {}
 
 pub type Result<T> = std::result::Result<T, TensorError>;
 

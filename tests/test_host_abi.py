@@ -247,6 +247,11 @@ def test_environment_defaults_are_read_by_the_library():
     code = "import fv_sdpa; l = fv_sdpa.lib(); print(l.fv_rt_log_level(), l.fv_vsa_default_sparsity())"
     assert _in_subprocess(code, {"FASTVIDEO_LOG": "debug", "FASTVIDEO_VSA_SPARSITY": " 0.875 "}) == "2 0.875"
     assert _in_subprocess(code, {"FASTVIDEO_LOG": "0", "FASTVIDEO_VSA_SPARSITY": "sparse"}) == "0 0.8"
+    # the reference trims, then parses with Rust's f64 grammar (settings/parse.rs:43-45): a leading '+' and
+    # exponents are numbers, hex floats and "nan(...)" (which strtod alone would take) are not
+    for text, want in ((" 0.5", "0.5"), ("+0.25", "0.25"), ("5e-1\n", "0.5"), ("0x1p-1", "0.8"), ("nan(1)", "0.8"),
+                       ("0.5 0.6", "0.8"), ("", "0.8")):
+        assert _in_subprocess(code, {"FASTVIDEO_LOG": "0", "FASTVIDEO_VSA_SPARSITY": text}) == "0 " + want, text
     env = {k: v for k, v in os.environ.items() if k not in ("FASTVIDEO_LOG", "FASTVIDEO_VSA_SPARSITY")}
     import subprocess
     import sys
@@ -254,3 +259,39 @@ def test_environment_defaults_are_read_by_the_library():
     r = subprocess.run([sys.executable, "-c", "import sys; sys.path[:0] = %r; " % [ROOT, os.path.join(ROOT, "fastvideo-rs_amd")]
                         + code], capture_output=True, text=True, env=env, timeout=120)
     assert r.stdout.strip() == "1 0.8", r.stderr[-500:]
+
+
+def test_static_splitkv_never_refuses_its_own_choice():
+    """fv_sdpa_dense_bf16_splitkv_static with splits == 0 runs the library's choice stepped down to what its
+    32 MiB buffer holds (host arithmetic: fv_sdpa_splitkv_static_splits); only an explicit count that cannot
+    fit is refused; absurd counts are settled, not divided by."""
+    lib = fv_sdpa.lib()
+    cap = lib.fv_sdpa_splitkv_static_bytes()
+    assert cap == 32 << 20
+    stepped = 0
+    for d in (128, 64):
+        for bh in (1, 2, 3, 4, 6, 8, 12, 16, 24, 40):
+            for sq in (1, 64, 256, 257, 512, 1024, 1560, 2048, 3000, 4096, 4680, 8192):
+                for sk in (64, 512, 1560, 4096, 4680, 16384, 32760, 75600):
+                    auto = lib.fv_sdpa_splitkv_static_splits(bh, sq, sk, d, 0)
+                    chosen = lib.fv_sdpa_splitkv_choose(bh, sq, sk)
+                    assert 1 <= auto <= chosen, (bh, sq, sk, d, auto, chosen)
+                    assert lib.fv_sdpa_splitkv_workspace_bytes(bh, sq, d, auto) <= cap
+                    if auto < chosen:
+                        stepped += 1
+                        nxt = auto + 1    # the next count that is a real split count does not fit
+                        while nxt <= chosen and lib.fv_sdpa_splitkv_static_splits(bh, sq, sk, d, nxt) == auto:
+                            nxt += 1
+                        assert nxt > chosen or lib.fv_sdpa_splitkv_static_splits(bh, sq, sk, d, nxt) == 0
+    assert stepped > 0
+    # the three shapes that used to be refused: 16 splits chosen, partials 262 144 bytes over the buffer
+    for bh, sq in ((1, 4096), (2, 2048), (4, 1024)):
+        assert lib.fv_sdpa_splitkv_choose(bh, sq, 32760) == 16
+        assert lib.fv_sdpa_splitkv_workspace_bytes(bh, sq, 128, 16) == 33816576 > cap
+        assert lib.fv_sdpa_splitkv_static_splits(bh, sq, 32760, 128, 0) == 15
+        assert lib.fv_sdpa_splitkv_static_splits(bh, sq, 32760, 128, 16) == 0     # explicit and too large: refused
+    # explicit counts: settled so that no split is empty, never more than the key tiles
+    assert lib.fv_sdpa_splitkv_static_splits(12, 256, 32760, 128, 7) == 7
+    assert lib.fv_sdpa_splitkv_static_splits(12, 256, 640, 128, 7) == 5            # 10 tiles / ceil(10 / 7) = 2 per split
+    assert lib.fv_sdpa_splitkv_static_splits(1, 256, 640, 128, 2 ** 64 - 1) == 10  # no wrap, no division by zero
+    assert lib.fv_sdpa_splitkv_static_splits(1, 256, 64, 128, 5) == 1

@@ -138,10 +138,87 @@ def test_python_loader_table_agrees_with_the_header():
 
 
 def test_committed_ffi_is_what_the_generator_writes(tmp_path):
-    committed = open(os.path.join(CRATE, "src", "ffi.rs")).read()
-    subprocess.check_call([sys.executable, os.path.join(CRATE, "gen_ffi.py")])
-    again = open(os.path.join(CRATE, "src", "ffi.rs")).read()
-    assert again == committed
+    path = os.path.join(CRATE, "src", "ffi.rs")
+    committed = open(path).read()
+    before = os.stat(path).st_mtime_ns
+    out = tmp_path / "ffi.rs"
+    subprocess.check_call([sys.executable, os.path.join(CRATE, "gen_ffi.py"), str(out)])
+    assert out.read_text() == committed
+    assert os.stat(path).st_mtime_ns == before   # the tracked file is compared with, never written
+
+
+def split_top_level(args):
+    """Comma-separated pieces of a Rust argument list, commas inside (), [], {}, <> or || closures kept."""
+    out, depth, cur, bars = [], 0, "", 0
+    for i, ch in enumerate(args):
+        if ch in "([{":
+            depth += 1
+        elif ch in ")]}":
+            depth -= 1
+        elif ch == "|" and depth == 0 and args[i - 1:i + 2] not in ("||",):
+            bars ^= 1
+        if ch == "," and depth == 0 and not bars:
+            out.append(cur.strip())
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip():
+        out.append(cur.strip())
+    return out
+
+
+def call_sites(src, prefix):
+    """(name, argument list) of every `prefix::name(...)` call in `src`, matching parentheses."""
+    sites = []
+    for m in re.finditer(re.escape(prefix) + r"::([a-zA-Z0-9_]+)\(", src):
+        depth, i = 1, m.end()
+        while depth:
+            depth += {"(": 1, ")": -1}.get(src[i], 0)
+            i += 1
+        sites.append((m.group(1), split_top_level(src[m.end():i - 1])))
+    return sites
+
+
+def test_every_ffi_call_site_passes_as_many_arguments_as_the_declaration_has():
+    src = re.sub(r"//[^\n]*", "", open(os.path.join(CRATE, "src", "lib.rs")).read())
+    _, rdecl = rust_declarations()
+    sites = call_sites(src, "ffi")
+    assert len(sites) >= 18
+    for name, args in sites:
+        assert name in rdecl, name
+        assert len(args) == len(rdecl[name][1]), (name, len(args), len(rdecl[name][1]), args)
+    # the HIP runtime calls of the crate against its own declarations (src/hip.rs)
+    hip = re.sub(r"//[^\n]*", "", open(os.path.join(CRATE, "src", "hip.rs")).read())
+    hdecl = {m.group(1): split_top_level(m.group(2)) for m in re.finditer(r"pub fn (hip[A-Za-z]+)\(([^)]*)\)", hip)}
+    hsites = [c for c in call_sites(src, "hip") if c[0].startswith("hip")]
+    assert len(hsites) >= 6
+    for name, args in hsites:
+        assert name in hdecl, name
+        assert len(args) == len(hdecl[name]), (name, args, hdecl[name])
+
+
+def test_shims_keep_the_reference_parameter_names_and_order():
+    """Parameter names, in order, of the reference's entries (crates/fastvideo-cudarc/src/rt/sdpa.rs:56-141,
+    attn.rs:225-231, 526-536, 652-659, vsa.rs:358-370; transcribed names only)."""
+    src = " ".join(re.sub(r"//[^\n]*", "", open(os.path.join(CRATE, "src", "lib.rs")).read()).split())
+    want = {
+        "sdpa": ["q", "k", "v", "plan"],
+        "device_mma_sdpa": ["q", "k", "v", "scale", "out_bf16"],
+        "device_mma_sdpa_causal": ["q", "k", "v", "scale", "out_bf16", "mask"],
+        "device_mma_sdpa_window": ["q", "k", "v", "scale", "out_bf16", "mask"],
+        "vsa_attention_device": ["q", "k", "v", "gate", "plan", "topk", "bh", "seq", "dim", "scale", "group"],
+        "dense": ["scale"], "masked": ["scale", "mask"], "fp8_first": ["self"], "composed": ["scale", "mask"],
+        "block_causal": ["scale", "mask"], "vdn_window": ["scale", "mask"], "kv_window": [], "kv_window_with": ["flash"],
+    }
+    # two deliberate differences: no `sm_major` (attn.rs:112-119: one architecture here), and the two fields
+    # `block_causal_for` reads from the model config (attn.rs:630-645) passed as plain numbers
+    want["mma_sdpa_supported"] = ["b", "h", "sq", "sk", "d"]
+    want["block_causal_for"] = ["num_frames_per_block", "local_attn_size", "frame_tokens"]
+    for name, params in want.items():
+        m = re.search(r"pub fn %s\(([^)]*)\)" % name, src)
+        assert m, name
+        got = [a.split(":")[0].strip() for a in split_top_level(m.group(1))]
+        assert got == params, (name, got)
 
 
 def test_shims_carry_the_reference_signatures():

@@ -76,6 +76,34 @@ def test_static_buffer_entry_equals_the_workspace_entry_on_two_calls_in_a_row(or
         assert_parity(got3.cpu().numpy(), oracle.sdpa_composed(q3, k3, v3), f"no_alloc_d64_splits{splits3}")
 
 
+def test_static_buffer_entry_steps_its_own_choice_down_to_what_fits(oracle):
+    """splits == 0 at a shape whose chosen count (16) would need 262 144 bytes more than the buffer holds:
+    the entry runs 15 splits instead of refusing, bit-identical to the workspace entry at 15."""
+    import torch
+
+    import fv_sdpa
+
+    lib = fv_sdpa.lib()
+    bh, sq, sk, d = 1, 4096, 32760, 128
+    assert int(lib.fv_sdpa_splitkv_choose(bh, sq, sk)) == 16
+    assert int(lib.fv_sdpa_splitkv_workspace_bytes(bh, sq, d, 16)) > int(lib.fv_sdpa_splitkv_static_bytes())
+    assert int(lib.fv_sdpa_splitkv_static_splits(bh, sq, sk, d, 0)) == 15
+    announce(f"no-alloc splitkv stepped-down choice bh={bh} sq={sq} sk={sk} seed=5400")
+    q, k, v = qkv(5400, bh, sq, sk, d)
+    tq, tk, tv = (to_dev_bf16(x) for x in (q, k, v))
+    stream = torch.cuda.current_stream().cuda_stream
+    got = torch.full((bh, sq, d), float("nan"), device="cuda")
+    rc = lib.fv_sdpa_dense_bf16_splitkv_static(tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), got.data_ptr(), 0, bh, sq, sk, d,
+                                               float(d) ** -0.5, 0, 0, 0, 0, stream)
+    assert rc == 0, lib.fv_sdpa_last_error().decode()
+    _, want = _both(lib, torch, tq, tk, tv, 15, False)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    rows = np.array([0, 1, 255, 256, 2047, sq - 1])
+    assert_parity(got[:, torch.from_numpy(rows).cuda()].cpu().numpy(), oracle.sdpa_composed_rows(q, k, v, rows),
+                  "no_alloc_stepped_down")
+
+
 def test_static_buffer_entry_refuses_what_does_not_fit():
     import torch
 
