@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(_PKG, "libfv_sdpa_hip.so")
+# FV_SDPA_HIP_LIB names another build of the same library (the host-sanitizer build of `make ubsan`)
+LIB_PATH = os.environ.get("FV_SDPA_HIP_LIB") or os.path.join(_PKG, "libfv_sdpa_hip.so")
 CSRC = os.path.join(_PKG, "csrc")
 
 FV_OK = 0

@@ -9,9 +9,7 @@ import pytest
 from util import ROOT
 
 
-@pytest.mark.skipif(shutil.which("gcc") is None, reason="no C compiler")
-def test_header_compiles_as_c_and_links(tmp_path):
-    pkg = os.path.join(ROOT, "fastvideo-rs_amd")
+def _host_calls(tmp_path, pkg):
     exe = str(tmp_path / "host_calls")
     subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
                            os.path.join(ROOT, "tests", "c_abi", "host_calls.c"), "-o", exe, "-L", pkg, "-lfv_sdpa_hip",
@@ -25,6 +23,38 @@ def test_header_compiles_as_c_and_links(tmp_path):
     assert "shards=0,6,6,5 " in line                 # rt/sp.rs:66-74
     assert "backend=1 route=2:1,2 " in line
     assert "local_attn_size=-1 keeps a 21-frame KV window" in line   # the refused plan's message
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="no C compiler")
+def test_header_compiles_as_c_and_links(tmp_path):
+    _host_calls(tmp_path, os.path.join(ROOT, "fastvideo-rs_amd"))
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None or shutil.which("hipcc") is None, reason="no compilers")
+def test_host_layer_is_clean_under_the_undefined_behaviour_sanitizer(tmp_path):
+    """`make ubsan` builds the library with its host code under -fsanitize=undefined in trap mode (device code
+    as always) into a temp dir; the C program above and every host-only test of the C ABI (geometry, KV-cache
+    plans, tile walks, routes, argument refusals, known answers) then run against that build in child
+    processes: undefined behaviour anywhere in the host layer kills the child with SIGILL."""
+    import sys
+
+    out = tmp_path / "ubsan"
+    csrc = os.path.join(ROOT, "fastvideo-rs_amd", "csrc")
+    b = subprocess.run(["make", "-C", csrc, "-j8", "ubsan", f"UBSAN_DIR={out}"], capture_output=True, text=True)
+    assert b.returncode == 0, b.stderr[-3000:]
+    so = out / "libfv_sdpa_hip.so"
+    assert so.exists()
+    dump = subprocess.run(["objdump", "-d", str(so)], capture_output=True, text=True).stdout
+    assert dump.count("ud1") + dump.count("ud2") > 100      # the traps are in: the flags reached the host pass
+    _host_calls(tmp_path, str(out))
+    env = dict(os.environ, FV_SDPA_HIP_LIB=str(so))
+    r = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-m", "not gpu", "-p", "no:cacheprovider",
+                        os.path.join(ROOT, "tests", "test_host_abi.py"),
+                        os.path.join(ROOT, "tests", "test_golden_known_answers.py"),
+                        os.path.join(ROOT, "tests", "test_oracle_kv_cache.py")],
+                       capture_output=True, text=True, env=env, cwd=ROOT, timeout=900)
+    assert r.returncode == 0, (r.returncode, r.stdout[-3000:], r.stderr[-2000:])
+    assert " passed" in r.stdout
 
 
 def test_oracle_c_functions_are_clean_under_address_and_undefined_sanitizers(tmp_path):
