@@ -32,17 +32,18 @@ namespace {
 int fail_hip(hipError_t e, const char* what) { return fv_fail_hip(e, what); }
 int decline(const char* why) { return fv_decline(why); }
 
+// y = bf16(x * mul), RNE; mul == 1 is the plain cast (x * 1.0f is x)
 __global__ void cast_f32_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y,
-                                     size_t n) {
+                                     size_t n, float mul) {
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i + 4 <= n && ((((uintptr_t)x) & 15) == 0) && ((((uintptr_t)y) & 7) == 0)) {
         const fv::f32x4 v = *reinterpret_cast<const fv::f32x4*>(x + i);
         fv::s16x4 o;
 #pragma unroll
-        for (int j = 0; j < 4; j++) o[j] = (short)fv::bf16_rne_bits(v[j]);
+        for (int j = 0; j < 4; j++) o[j] = (short)fv::bf16_rne_bits(v[j] * mul);
         *reinterpret_cast<fv::s16x4*>(y + i) = o;
     } else {
-        for (size_t j = i; j < n && j < i + 4; j++) y[j] = fv::bf16_rne_bits(x[j]);
+        for (size_t j = i; j < n && j < i + 4; j++) y[j] = fv::bf16_rne_bits(x[j] * mul);
     }
 }
 
@@ -353,15 +354,19 @@ int fv_sdpa_vdn_window_bf16(const uint16_t* q, const uint16_t* k, const uint16_t
     return flash_common(q, k, v, out, out_is_bf16, bh, sq, sk, d, scale, m, stream);
 }
 
-int fv_cast_f32_bf16(const float* x, uint16_t* y, size_t n, void* stream) {
+int fv_cast_f32_bf16_scaled(const float* x, uint16_t* y, size_t n, float mul, void* stream) {
     if (n == 0) return FV_OK;
     const size_t threads = (n + 3) / 4;
     const size_t blocks = (threads + 255) / 256;
     if (blocks > (size_t)INT_MAX) return decline("cast: too many elements for one launch");
     hipLaunchKernelGGL(cast_f32_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0,
-                       (hipStream_t)stream, x, y, n);
+                       (hipStream_t)stream, x, y, n, mul);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? FV_OK : fail_hip(e, "cast_f32_bf16");
+}
+
+int fv_cast_f32_bf16(const float* x, uint16_t* y, size_t n, void* stream) {
+    return fv_cast_f32_bf16_scaled(x, y, n, 1.0f, stream);
 }
 
 int fv_cast_bf16_f32(const uint16_t* x, float* y, size_t n, void* stream) {

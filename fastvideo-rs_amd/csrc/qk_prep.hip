@@ -77,7 +77,7 @@ template <bool X16, bool W16, bool ROUND16, int NC>
 __global__ __launch_bounds__(256) void qk_norm_rope_bhsd_kernel(
     const void* __restrict__ src, const void* __restrict__ w, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, void* __restrict__ out, long rows, int seq, int heads, int d,
-    long src_width, long col_off, float eps, const unsigned* __restrict__ row_map, long out_rows) {
+    long src_width, long col_off, float eps, float out_mul, const unsigned* __restrict__ row_map, long out_rows) {
 #pragma clang fp contract(off)
     const int lane = threadIdx.x & 63;
     const long row = (long)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
@@ -160,6 +160,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_bhsd_kernel(
                 r[i + 1] = ROUND16 ? (x2 * cv + x1 * sv) : (x1 * sv + x2 * cv);
             }
         }
+        // the caller's output factor (1 = none: x * 1.0f is x), before the one rounding of the rotated values
+#pragma unroll
+        for (int i = 0; i < 8; i++) r[i] = r[i] * out_mul;
         const size_t o = (((size_t)b * heads + h) * out_rows + orow) * d + p;
         if constexpr (ROUND16) {
             *reinterpret_cast<u32x4*>((unsigned short*)out + o) = pack_bf16x8(r);
@@ -219,18 +222,18 @@ __global__ __launch_bounds__(256) void merge_heads_kernel(const u32x4* __restric
 template <bool X16, bool W16, bool R16, int NC>
 void launch_qk_nc(dim3 grid, hipStream_t st, const void* src, const void* w, const float* cos_t,
                   const float* sin_t, void* out, long rows, int seq, int heads, int d, long src_width,
-                  long col_off, float eps, const unsigned* row_map, long out_rows) {
+                  long col_off, float eps, float out_mul, const unsigned* row_map, long out_rows) {
     hipLaunchKernelGGL((qk_norm_rope_bhsd_kernel<X16, W16, R16, NC>), grid, dim3(256), 0, st, src, w, cos_t, sin_t,
-                       out, rows, seq, heads, d, src_width, col_off, eps, row_map, out_rows);
+                       out, rows, seq, heads, d, src_width, col_off, eps, out_mul, row_map, out_rows);
 }
 
 template <bool X16, bool W16, bool R16>
 void launch_qk_r(const void* src, const void* w, const float* cos_t, const float* sin_t, void* out, long rows,
-                 int seq, int heads, int d, long src_width, long col_off, float eps, const unsigned* row_map,
-                 long out_rows, hipStream_t st) {
+                 int seq, int heads, int d, long src_width, long col_off, float eps, float out_mul,
+                 const unsigned* row_map, long out_rows, hipStream_t st) {
     const dim3 grid((unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock));
     const int per_lane = (heads * d / 8 + 63) / 64;   // 16-byte chunks per lane
-#define FV_QK_ARGS grid, st, src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, row_map, out_rows
+#define FV_QK_ARGS grid, st, src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, out_mul, row_map, out_rows
     if (per_lane <= 2) launch_qk_nc<X16, W16, R16, 2>(FV_QK_ARGS);
     else if (per_lane <= 3) launch_qk_nc<X16, W16, R16, 3>(FV_QK_ARGS);        // 12 heads x 128
     else if (per_lane <= 6) launch_qk_nc<X16, W16, R16, 6>(FV_QK_ARGS);
@@ -242,12 +245,12 @@ void launch_qk_r(const void* src, const void* w, const float* cos_t, const float
 template <bool X16, bool W16>
 hipError_t launch_qk(int round16, const void* src, const void* w, const float* cos_t, const float* sin_t,
                      void* out, long rows, int seq, int heads, int d, long src_width, long col_off,
-                     float eps, const unsigned* row_map, long out_rows, hipStream_t st) {
+                     float eps, float out_mul, const unsigned* row_map, long out_rows, hipStream_t st) {
     if (round16)
-        launch_qk_r<X16, W16, true>(src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, row_map,
-                                    out_rows, st);
+        launch_qk_r<X16, W16, true>(src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, out_mul,
+                                    row_map, out_rows, st);
     else
-        launch_qk_r<X16, W16, false>(src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps,
+        launch_qk_r<X16, W16, false>(src, w, cos_t, sin_t, out, rows, seq, heads, d, src_width, col_off, eps, out_mul,
                                      row_map, out_rows, st);
     return hipGetLastError();
 }
@@ -260,9 +263,10 @@ extern "C" {
 static int qk_norm_rope_common(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
                                const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
                                size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
-                               size_t col_off, float eps, const uint32_t* row_map, size_t out_rows,
+                               size_t col_off, float eps, float out_mul, const uint32_t* row_map, size_t out_rows,
                                void* stream) {
     if (!src || !w || !out) return fv_invalid("qk_norm_rope: null operand");
+    if (!(out_mul == out_mul) || out_mul - out_mul != 0.0f) return fv_invalid("qk_norm_rope: out_mul must be finite");
     if ((cos_t == nullptr) != (sin_t == nullptr)) return fv_invalid("qk_norm_rope: one rope table without the other");
     if (batch == 0 || seq == 0) return FV_OK;
     if (heads == 0 || d == 0 || col_off + heads * d > src_width)
@@ -278,7 +282,7 @@ static int qk_norm_rope_common(const void* src, int src_is_bf16, const void* w, 
     hipError_t e;
 #define FV_QK_CALL(X16, W16)                                                                                  \
     fv::launch_qk<X16, W16>(out_is_bf16, src, w, cos_t, sin_t, out, rows, (int)seq, (int)heads, (int)d,        \
-                            (long)src_width, (long)col_off, eps, row_map, (long)out_rows, st)
+                            (long)src_width, (long)col_off, eps, out_mul, row_map, (long)out_rows, st)
     if (src_is_bf16 && w_is_bf16) e = FV_QK_CALL(true, true);
     else if (src_is_bf16) e = FV_QK_CALL(true, false);
     else if (w_is_bf16) e = FV_QK_CALL(false, true);
@@ -290,20 +294,20 @@ static int qk_norm_rope_common(const void* src, int src_is_bf16, const void* w, 
 int fv_qk_norm_rope_bhsd(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
                          const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
                          size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
-                         size_t col_off, float eps, void* stream) {
+                         size_t col_off, float eps, float out_mul, void* stream) {
     return qk_norm_rope_common(src, src_is_bf16, w, w_is_bf16, cos_t, sin_t, out, out_is_bf16, batch, seq, heads, d,
-                               src_width, col_off, eps, nullptr, seq, stream);
+                               src_width, col_off, eps, out_mul, nullptr, seq, stream);
 }
 
 int fv_qk_norm_rope_tiles(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
                           const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
                           size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
-                          size_t col_off, float eps, const uint32_t* token_slot, size_t padded,
+                          size_t col_off, float eps, float out_mul, const uint32_t* token_slot, size_t padded,
                           void* stream) {
     if (!token_slot) return fv_invalid("qk_norm_rope_tiles: null token_slot");
     if (padded < seq) return fv_invalid("qk_norm_rope_tiles: padded < seq");
     return qk_norm_rope_common(src, src_is_bf16, w, w_is_bf16, cos_t, sin_t, out, out_is_bf16, batch, seq, heads, d,
-                               src_width, col_off, eps, token_slot, padded, stream);
+                               src_width, col_off, eps, out_mul, token_slot, padded, stream);
 }
 
 static int split_heads_common(const void* src, void* out, int is_bf16, size_t batch, size_t seq, size_t heads,

@@ -123,6 +123,7 @@ TensorError msg(std::string s) { return TensorError{std::move(s)}; }
 std::atomic<uint64_t> g_fused{0}, g_causal{0}, g_composed{0}, g_cast{0}, g_masks{0};
 thread_local std::optional<bool> g_bf16_override;
 thread_local std::optional<Backend> g_backend_override;
+thread_local std::optional<bool> g_fold_override;
 
 // rt/sdpa.rs:234-246 `retired`
 std::string retired(Backend b) {
@@ -176,13 +177,14 @@ std::string rc_message(int rc) {
     return std::string(fv_sdpa_last_error()) + " (rc " + std::to_string(rc) + ")";
 }
 
-// A bf16 view of `x`: `x` itself when it already is bf16, else a rounded copy in `tmp`.
-Result<const Tensor*> as_bf16(const Tensor& x, Tensor& tmp, hipStream_t st) {
+// A bf16 view of `x`: `x` itself when it already is bf16, else a rounded copy in `tmp` (of x * mul: the
+// product in f32, one rounding).
+Result<const Tensor*> as_bf16(const Tensor& x, Tensor& tmp, hipStream_t st, float mul = 1.0f) {
     if (x.dtype == DType::Bf16) return &x;
     auto r = Tensor::alloc(x.shape, DType::Bf16, st);
     if (!is_ok(r)) return std::get<TensorError>(r);
     tmp = std::move(std::get<Tensor>(r));
-    const int rc = fv_cast_f32_bf16((const float*)x.data, (uint16_t*)tmp.data, x.numel(), st);
+    const int rc = fv_cast_f32_bf16_scaled((const float*)x.data, (uint16_t*)tmp.data, x.numel(), mul, st);
     if (rc != FV_OK) return TensorError{"cast_f32_bf16: " + rc_message(rc), rc < 0 ? -rc : 0};
     g_cast++;
     return &tmp;
@@ -246,8 +248,19 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
                                     const VdnWindow* window = nullptr) {
     const auto s = bhsd(q, k, v);
     if (!s || !fv_sdpa_supported(s->b, s->h, s->sq, s->sk, s->d)) return std::optional<Tensor>{};
+    // f32 queries are rounded to bf16 here, once: with the fold switch on, of q * (scale * log2(e)), and the
+    // kernel then runs at scale = ln 2, its form without the per-score multiply-add
+    float sc = default_scale(scale, s->d);
+    float q_mul = 1.0f;
+    if (q.dtype == DType::F32 && fold_scale()) {
+        const float c = sc * 1.4426950408889634f;
+        if (c > 0.0f && c < 3.0e38f && !fv_sdpa_is_log2_domain_scale(sc)) {
+            q_mul = c;
+            sc = FV_SDPA_SCALE_LOG2_DOMAIN;
+        }
+    }
     Tensor tq, tk, tv;
-    auto rq = as_bf16(q, tq, st);
+    auto rq = as_bf16(q, tq, st, q_mul);
     if (!is_ok(rq)) return std::get<TensorError>(rq);
     auto rk = as_bf16(k, tk, st);
     if (!is_ok(rk)) return std::get<TensorError>(rk);
@@ -259,7 +272,6 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
     const auto* pq = (const uint16_t*)std::get<const Tensor*>(rq)->data;
     const auto* pk = (const uint16_t*)std::get<const Tensor*>(rk)->data;
     const auto* pv = (const uint16_t*)std::get<const Tensor*>(rv)->data;
-    const float sc = default_scale(scale, s->d);
     int rc;
     if (causal)
         rc = fv_sdpa_block_causal_bf16(pq, pk, pv, out.data, out_bf16, s->b * s->h, s->sq, s->sk, s->d, sc,
@@ -535,6 +547,12 @@ bool causal_flash_enabled() {
     static const bool env = env_flag("FASTVIDEO_WAN_CAUSAL_FLASH", true);
     return env;
 }
+bool fold_scale() {
+    if (g_fold_override) return *g_fold_override;
+    static const bool env = env_flag("FASTVIDEO_SDPA_FOLD_SCALE", true);
+    return env;
+}
+void set_fold_scale_override(std::optional<bool> v) { g_fold_override = v; }
 
 Backend parse_backend(const std::string& v) {
     if (v == "cublas") return Backend::Cublas;
@@ -745,6 +763,10 @@ void fv_rt_set_bf16_activations(int v) {
     fv::rt::set_bf16_activations_override(v < 0 ? std::nullopt : std::optional<bool>(v != 0));
 }
 int fv_rt_bf16_activations(void) { return fv::rt::bf16_activations() ? 1 : 0; }
+void fv_rt_set_fold_scale(int v) {
+    fv::rt::set_fold_scale_override(v < 0 ? std::nullopt : std::optional<bool>(v != 0));
+}
+int fv_rt_fold_scale(void) { return fv::rt::fold_scale() ? 1 : 0; }
 
 int fv_rt_log_level(void) { return fv::rt::log_level(); }
 int fv_rt_parse_log_level(const char* v) { return fv::rt::log_level_from(v); }

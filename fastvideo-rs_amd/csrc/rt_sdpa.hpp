@@ -109,6 +109,10 @@ bool bf16_activations();
 void set_bf16_activations_override(std::optional<bool> v);
 // rt/sdpa_rule.rs `causal_flash_enabled`: FASTVIDEO_WAN_CAUSAL_FLASH, default on.
 bool causal_flash_enabled();
+// Whether the bf16 copy the library makes of an f32 q carries scale * log2(e) (one rounding of the product; the
+// fused kernel then runs at scale = ln 2): FASTVIDEO_SDPA_FOLD_SCALE, default on, overridable per thread.
+bool fold_scale();
+void set_fold_scale_override(std::optional<bool> v);
 
 // rt/sdpa_rule.rs:178-219 `Backend` / `parse_backend` / `backend`: FASTVIDEO_SDPA (lower-cased,
 // read once), overridable per thread. Anything but the four names below is the dense default.

@@ -55,6 +55,7 @@ SIGNATURES = {
     "fv_sdpa_block_causal_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float,
                                             _sz, _sz, _sz, _vp]),
     "fv_cast_f32_bf16": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "fv_cast_f32_bf16_scaled": (C.c_int, [_vp, _vp, _sz, C.c_float, _vp]),
     "fv_softmax_last": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _vp]),
     "fv_cast_bf16_f32": (C.c_int, [_vp, _vp, _sz, _vp]),
     "fv_sdpa_composed_f32": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _vp, _sz, _sz, _sz, _sz, C.c_float, _vp]),
@@ -63,6 +64,8 @@ SIGNATURES = {
     "fv_rt_free": (C.c_int, [_vp, _vp]),
     "fv_rt_set_bf16_activations": (None, [C.c_int]),
     "fv_rt_bf16_activations": (C.c_int, []),
+    "fv_rt_set_fold_scale": (None, [C.c_int]),
+    "fv_rt_fold_scale": (C.c_int, []),
     "fv_rt_stats": (None, [_vp]),
     "fv_rt_log_level": (C.c_int, []),
     "fv_rt_parse_log_level": (C.c_int, [C.c_char_p]),
@@ -95,11 +98,11 @@ SIGNATURES = {
     "fv_vdn_window_allows": (C.c_int, [_sz, _sz, _sz, _sz, _sz, _sz, _sz]),
     "fv_vdn_window_dense_mask": (None, [_sz, _sz, _sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_qk_norm_rope_bhsd": (C.c_int, [_vp, C.c_int, _vp, C.c_int, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz,
-                                       _sz, C.c_float, _vp]),
+                                       _sz, C.c_float, C.c_float, _vp]),
     "fv_split_heads_bhsd": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz, _sz, _vp]),
     "fv_merge_heads": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _vp]),
     "fv_qk_norm_rope_tiles": (C.c_int, [_vp, C.c_int, _vp, C.c_int, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz,
-                                        _sz, C.c_float, _vp, _sz, _vp]),
+                                        _sz, C.c_float, C.c_float, _vp, _sz, _vp]),
     "fv_split_heads_tiles": (C.c_int, [_vp, _vp, C.c_int, _sz, _sz, _sz, _sz, _sz, _sz, _vp, _sz, _vp]),
 }
 

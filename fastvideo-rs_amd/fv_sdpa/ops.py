@@ -121,10 +121,14 @@ def sdpa_vdn_window_bf16(q, k, v, video_start, frame_tokens, frames, chunk=0, ra
     return out
 
 
-def cast_f32_bf16(x):
+def cast_f32_bf16(x, mul=None):
+    """bf16(x) (RNE), or bf16(x * mul) with the product in f32."""
     _need(x, torch.float32, "x")
     y = torch.empty(x.shape, device=x.device, dtype=torch.bfloat16)
-    _lib.check(_lib.lib().fv_cast_f32_bf16(x.data_ptr(), y.data_ptr(), x.numel(), _stream()))
+    if mul is None:
+        _lib.check(_lib.lib().fv_cast_f32_bf16(x.data_ptr(), y.data_ptr(), x.numel(), _stream()))
+    else:
+        _lib.check(_lib.lib().fv_cast_f32_bf16_scaled(x.data_ptr(), y.data_ptr(), x.numel(), float(mul), _stream()))
     return y
 
 

@@ -23,11 +23,13 @@ def _is16(t, name):
     raise ValueError(f"{name}: want f32 or bf16")
 
 
-def qk_norm_rope_bhsd(proj, col_off, heads, weight, rope=None, eps=1e-6, out_bf16=None, tiles=None, out=None):
+def qk_norm_rope_bhsd(proj, col_off, heads, weight, rope=None, eps=1e-6, out_bf16=None, tiles=None, out=None,
+                      out_mul=1.0):
     """proj [batch, seq, width] -> [batch, heads, seq, d]. out_bf16 (default: proj is bf16)
     selects the bf16 kernel with its rounding points; otherwise the f32 op. `tiles` (a VsaCtx): the
     head planes are written in the plan's tile-slot order, [batch, heads, padded, d], padding zero
-    (`out`: a buffer from an earlier call, whose padding rows are zero already)."""
+    (`out`: a buffer from an earlier call, whose padding rows are zero already). `out_mul`: a factor on
+    every output value, applied in f32 before the write (scale * log2(e) for an SDPA call at ln 2)."""
     batch, seq, width = proj.shape
     if tiles is not None and seq != tiles.seq:
         raise ValueError(f"qk norm: proj has {seq} tokens, the tile plan {tiles.seq}")
@@ -54,19 +56,21 @@ def qk_norm_rope_bhsd(proj, col_off, heads, weight, rope=None, eps=1e-6, out_bf1
                                                     cos.data_ptr() if cos is not None else None,
                                                     sin.data_ptr() if sin is not None else None, out.data_ptr(),
                                                     int(out_bf16), batch, seq, heads, d, width, col_off, eps,
-                                                    tiles.token_slot.data_ptr(), tiles.padded, _stream()))
+                                                    float(out_mul), tiles.token_slot.data_ptr(), tiles.padded,
+                                                    _stream()))
         return out
     out = torch.empty((batch, heads, seq, d), device=proj.device, dtype=odt)
     _lib.check(_lib.lib().fv_qk_norm_rope_bhsd(proj.data_ptr(), x16, weight.data_ptr(), w16,
                                                cos.data_ptr() if cos is not None else None,
                                                sin.data_ptr() if sin is not None else None, out.data_ptr(),
-                                               int(out_bf16), batch, seq, heads, d, width, col_off, eps, _stream()))
+                                               int(out_bf16), batch, seq, heads, d, width, col_off, eps,
+                                               float(out_mul), _stream()))
     return out
 
 
-def qk_norm_rope_tiles(proj, col_off, heads, weight, ctx, rope=None, eps=1e-6, out_bf16=None, out=None):
+def qk_norm_rope_tiles(proj, col_off, heads, weight, ctx, rope=None, eps=1e-6, out_bf16=None, out=None, out_mul=1.0):
     """`qk_norm_rope_bhsd` writing VSA's tile-slot order directly (ctx: a VsaCtx)."""
-    return qk_norm_rope_bhsd(proj, col_off, heads, weight, rope, eps, out_bf16, tiles=ctx, out=out)
+    return qk_norm_rope_bhsd(proj, col_off, heads, weight, rope, eps, out_bf16, tiles=ctx, out=out, out_mul=out_mul)
 
 
 def split_heads_tiles(proj, col_off, heads, d, ctx, out=None):

@@ -9,7 +9,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["Plan", "BlockCausal", "VdnWindow", "sdpa", "with_bf16_act", "bf16_activations", "rt_stats", "TensorError",
+__all__ = ["Plan", "BlockCausal", "VdnWindow", "sdpa", "with_bf16_act", "bf16_activations", "with_fold_scale", "fold_scale", "rt_stats", "TensorError",
            "BACKENDS", "STEPS", "parse_backend", "backend", "with_backend", "shape_of", "dense_route"]
 
 
@@ -227,6 +227,22 @@ def with_bf16_act(on):
         yield
     finally:
         lib.fv_rt_set_bf16_activations(-1)
+
+
+def fold_scale():
+    return bool(_lib.lib().fv_rt_fold_scale())
+
+
+@contextmanager
+def with_fold_scale(on):
+    """Per-thread override of FASTVIDEO_SDPA_FOLD_SCALE: whether `sdpa` folds scale * log2(e) into the one
+    rounding of an f32 q (and runs the kernel at scale = ln 2)."""
+    lib = _lib.lib()
+    lib.fv_rt_set_fold_scale(int(bool(on)))
+    try:
+        yield
+    finally:
+        lib.fv_rt_set_fold_scale(-1)
 
 
 def rt_stats():

@@ -137,6 +137,10 @@ int fv_sdpa_vdn_window_bf16(const uint16_t* q, const uint16_t* k, const uint16_t
 /* rt/ops.rs:258-265 `cast_f32_bf16_device` + kernels/core.cu:121: f32 -> bf16
  * bits, RNE, NaN quiet, overflow to inf (kernels/core.cu:6-15). */
 int fv_cast_f32_bf16(const float* x, uint16_t* y, size_t n, void* stream);
+/* No counterpart in the reference: y = bf16(x * mul), the product in f32, one RNE rounding to bf16. With
+ * mul = scale * log2(e) this is Q for a call at FV_SDPA_SCALE_LOG2_DOMAIN: the softmax scale goes into Q
+ * before Q's only rounding to bf16 (fv_rt_sdpa does this by itself for f32 queries). */
+int fv_cast_f32_bf16_scaled(const float* x, uint16_t* y, size_t n, float mul, void* stream);
 /* bf16 bits -> f32 (exact widening), rt/tensor.rs `to_f32_act`. */
 int fv_cast_bf16_f32(const uint16_t* x, float* y, size_t n, void* stream);
 
@@ -197,6 +201,15 @@ int fv_rt_free(void* p, void* stream);
 /* rt/tensor.rs `with_bf16_act`: per-thread override of FASTVIDEO_BF16_ACT; v < 0 clears it. */
 void fv_rt_set_bf16_activations(int v);
 int fv_rt_bf16_activations(void);
+/* No counterpart in the reference. When q arrives as f32, fv_rt_sdpa itself makes the bf16 copy the fused
+ * kernels read (rt/sdpa.rs:167-181 `act16_operands`, rt/attn.rs:283-300): with this switch on (the default;
+ * FASTVIDEO_SDPA_FOLD_SCALE=0 turns it off, fv_rt_set_fold_scale overrides per thread, v < 0 clears) that one
+ * rounding is taken of q * (scale * log2(e)) and the kernel runs at FV_SDPA_SCALE_LOG2_DOMAIN, the form without
+ * the per-score multiply-add. Q is still rounded once, from the same f32 values, so the result is as close to
+ * the f32 host math as with the switch off (bf16(c q) in place of c bf16(q): different last bits, same error
+ * size); bf16 queries are never touched. Off reproduces the reference's order (round, then scale) exactly. */
+void fv_rt_set_fold_scale(int v);
+int fv_rt_fold_scale(void);
 /* rt/log.rs:17-37: the level FASTVIDEO_LOG selects (read once): 0 quiet ("0", "off", "false", "quiet",
  * "error"), 2 debug ("2", "debug", "trace", "verbose"), 1 info (unset or anything else). At info and above
  * fv_rt_sdpa writes one "[fastvideo] sdpa: <kernel> B= H= Sq= Sk= D=" line to stderr the first time a
@@ -388,18 +401,23 @@ int fv_vsa_attention_tiled(const uint16_t* qt, const uint16_t* kt, const uint16_
  *   rt/fuse/policy.rs:404-412, host twin rt/fuse/host.rs:217-276).
  * src and w are f32 or bf16 (flags); cos_t / sin_t are f32 [seq, d] (cos read from the even slot
  * of a pair, sin from the odd one) or both NULL for no rotation. Declines unless d, col_off and
- * src_width are multiples of 8. */
+ * src_width are multiples of 8.
+ * out_mul (no counterpart in the reference; 1.0f = the reference's op, bit for bit): every output value is
+ * multiplied by it in f32 after the rotation and before the write (before the ONE rounding of the bf16 form's
+ * rotated values), so q can leave the producer as q * scale * log2(e) for an SDPA call at
+ * FV_SDPA_SCALE_LOG2_DOMAIN without touching the norm weights. (Without rotation the bf16 form's value is
+ * already a bf16 number when out_mul meets it: a second rounding, to be weighed by the caller.) */
 int fv_qk_norm_rope_bhsd(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
                          const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
                          size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
-                         size_t col_off, float eps, void* stream);
+                         size_t col_off, float eps, float out_mul, void* stream);
 /* The same op writing VSA's tile-slot order: head planes are [padded, d] and token s lands in row
  * token_slot[s] (fv_vsa_tile_plan; every value < padded, others are skipped). Padding rows are not
  * written: zero `out` once, no call touches them afterwards. Feeds fv_vsa_attention_tiled. */
 int fv_qk_norm_rope_tiles(const void* src, int src_is_bf16, const void* w, int w_is_bf16,
                           const float* cos_t, const float* sin_t, void* out, int out_is_bf16,
                           size_t batch, size_t seq, size_t heads, size_t d, size_t src_width,
-                          size_t col_off, float eps, const uint32_t* token_slot, size_t padded,
+                          size_t col_off, float eps, float out_mul, const uint32_t* token_slot, size_t padded,
                           void* stream);
 /* rt/ops.rs:574-602 / kernels/core.cu:415-427 `split_heads_bhsd`: the value heads, a pure permute
  * of f32 or bf16 elements. */

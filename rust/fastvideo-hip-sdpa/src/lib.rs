@@ -447,15 +447,27 @@ fn fused(q: &CudaTensor, k: &CudaTensor, v: &CudaTensor, scale: Option<f32>, out
     if !mma_sdpa_supported(b, h, sq, sk, d) {
         return Ok(None);
     }
-    // the fused kernels read bf16; f32 operands are rounded once (RNE), as the reference does
+    // the fused kernels read bf16; f32 operands are rounded once (RNE), as the reference does. An f32 q is
+    // rounded as q * (scale * log2(e)) and the kernel then runs at ln 2, its form without the per-score
+    // multiply-add (fv_rt_fold_scale: on unless FASTVIDEO_SDPA_FOLD_SCALE=0).
+    let mut scale = scale.unwrap_or(1.0 / (d as f32).sqrt());
+    let mut q_mul = 1.0f32;
+    // SAFETY: reads a per-thread flag / host arithmetic only.
+    if q.dtype == TensorDType::F32 && unsafe { ffi::fv_rt_fold_scale() != 0 && ffi::fv_sdpa_is_log2_domain_scale(scale) == 0 } {
+        let c = scale * std::f32::consts::LOG2_E;
+        if c > 0.0 && c < 3.0e38 {
+            q_mul = c;
+            scale = ffi::FV_SDPA_SCALE_LOG2_DOMAIN;
+        }
+    }
     let (tq, tk, tv);
-    let as_bf16 = |t: &CudaTensor| -> Result<Option<CudaTensor>> {
+    let as_bf16 = |t: &CudaTensor, mul: f32| -> Result<Option<CudaTensor>> {
         if t.dtype == TensorDType::Bf16 {
             return Ok(None);
         }
         let c = HipTensor::alloc(t.shape.clone(), TensorDType::Bf16)?;
         // SAFETY: both buffers hold numel() elements on the current device.
-        let rc = unsafe { ffi::fv_cast_f32_bf16(t.device_ptr().cast_const().cast(), c.device_ptr().cast(), t.numel(), stream()) };
+        let rc = unsafe { ffi::fv_cast_f32_bf16_scaled(t.device_ptr().cast_const().cast(), c.device_ptr().cast(), t.numel(), mul, stream()) };
         if rc != FV_OK {
             return Err(msg(last_error()));
         }
@@ -469,15 +481,14 @@ fn fused(q: &CudaTensor, k: &CudaTensor, v: &CudaTensor, scale: Option<f32>, out
             return Ok(None);
         }
     }
-    tq = as_bf16(q)?;
-    tk = as_bf16(k)?;
-    tv = as_bf16(v)?;
+    tq = as_bf16(q, q_mul)?;
+    tk = as_bf16(k, 1.0)?;
+    tv = as_bf16(v, 1.0)?;
     let (pq, pk, pv) = (
         tq.as_ref().unwrap_or(q).device_ptr().cast_const().cast::<u16>(),
         tk.as_ref().unwrap_or(k).device_ptr().cast_const().cast::<u16>(),
         tv.as_ref().unwrap_or(v).device_ptr().cast_const().cast::<u16>(),
     );
-    let scale = scale.unwrap_or(1.0 / (d as f32).sqrt());
     let out = HipTensor::alloc(vec![b, h, sq, d], if out_bf16 { TensorDType::Bf16 } else { TensorDType::F32 })?;
     let st = stream();
     // SAFETY: operand pointers address [b*h, s, d] bf16 planes, `out` the [b*h, sq, d] result.

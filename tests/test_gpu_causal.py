@@ -9,7 +9,7 @@ dense kernel.
 import numpy as np
 import pytest
 
-from util import announce, assert_parity, qkv, sample_rows, to_dev_bf16
+from util import REL_L2_F32_OUT, announce, assert_parity, qkv, sample_rows, to_dev_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -152,7 +152,8 @@ def test_headline_causal_shape_sampled_rows(fv, oracle, bt):
     rows = sample_rows(3, s, 512, extra=[0, 255, 256, 10 * bt + 5, s - 1] + edges)
     assert rows.size >= 512 and set(edges) <= set(rows.tolist())
     want = oracle.sdpa_composed_rows(qn, kn, vn, rows, mask_bc=(bt, 0, 0))
-    assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, f"causal_headline_{bt}_{rows.size}_rows")
+    assert_parity(out[:, torch.from_numpy(rows).cuda()].cpu().numpy(), want, f"causal_headline_{bt}_{rows.size}_rows",
+                  max_rel_l2=REL_L2_F32_OUT)
     # the bf16 output is the RNE rounding of the f32 output, every element
     assert torch.equal(fv.sdpa_block_causal_bf16(q, k, v, bt, 0, 0, out_bf16=True), out.to(torch.bfloat16))
 

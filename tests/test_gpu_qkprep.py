@@ -99,6 +99,56 @@ def test_bf16_kernel_rounding_points(fv, oracle, case, rope, w16):
         assert u.max() <= 2, f"max ulp {u.max()}"
 
 
+@pytest.mark.parametrize("case", CASES[1:3])
+def test_out_mul_meets_the_values_before_their_one_rounding(fv, oracle, case):
+    """`out_mul` (scale * log2(e) for an SDPA call at ln 2): the f32 op's outputs times the factor; the bf16 kernel's
+    rotated f32 values times the factor, THEN the one rounding. The expected bf16 values are built here from the
+    oracle's un-rotated rows (already bf16 numbers: round_weighted) with numpy's unfused f32 arithmetic; at factor 1
+    that construction must be the oracle's own rotated output bit for bit, which pins it. A power-of-two factor
+    scales the plain output exactly; 1.0 is the plain output bit for bit."""
+    import torch
+
+    batch, seq, heads, d, extra, col_off = case
+    announce(f"qk_norm_rope out_mul {case}")
+    proj, w, cos, sin = _inputs(18, batch, seq, heads, d, extra, col_off)
+    dev = lambda a: torch.from_numpy(a).cuda()  # noqa: E731
+    c = np.float32(np.float32(1.0 / np.sqrt(d)) * np.float32(1.4426950408889634))
+    # f32 op
+    want32 = oracle.qk_norm_rope_bhsd(proj, col_off, heads, w, (cos, sin), 1e-6)
+    got32 = fv.qk_norm_rope_bhsd(dev(proj), col_off, heads, dev(w), (dev(cos), dev(sin)), 1e-6, out_mul=float(c))
+    plain32 = fv.qk_norm_rope_bhsd(dev(proj), col_off, heads, dev(w), (dev(cos), dev(sin)), 1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(got32, plain32 * float(c))               # one f32 multiply of the op's own output
+    assert np.abs(got32.cpu().numpy() - want32 * c).max() <= 2e-6 * max(1.0, np.abs(want32).max())
+    # bf16 kernel
+    p16 = oracle.quantize_bf16(proj)
+    n = oracle.wan_qk_norm_rope16(p16, col_off, heads, w, None, 1e-6)          # [b, h, s, d] bf16 numbers
+    x1, x2 = n[..., 0::2], n[..., 1::2]
+    cv, sv = cos[None, None, :, 0::2], sin[None, None, :, 1::2]
+
+    def expected(f):
+        rot = np.empty_like(n)
+        rot[..., 0::2] = x1 * cv - x2 * sv                                     # numpy f32: products and sums unfused
+        rot[..., 1::2] = x2 * cv + x1 * sv
+        return oracle.quantize_bf16(rot * np.float32(f))
+
+    assert np.array_equal(expected(1.0), oracle.wan_qk_norm_rope16(p16, col_off, heads, w, (cos, sin), 1e-6))
+    args = (dev(p16).to(torch.bfloat16), col_off, heads, dev(w), (dev(cos), dev(sin)), 1e-6)
+    plain = fv.qk_norm_rope_bhsd(*args)
+    assert torch.equal(fv.qk_norm_rope_bhsd(*args, out_mul=1.0), plain)
+    assert torch.equal(fv.qk_norm_rope_bhsd(*args, out_mul=0.25).float(), plain.float() * 0.25)
+    got = fv.qk_norm_rope_bhsd(*args, out_mul=float(c)).float().cpu().numpy()
+    want = expected(c)
+    u = _ulps(got, want, oracle)
+    assert (u != 0).mean() < 1e-3, f"fraction differing {(u != 0).mean()}"
+    assert np.abs(got - want).max() <= 0.03 * float(c)
+    # and it is NOT the twice-rounded value for a visible share of the elements (the test can tell the two apart)
+    twice = oracle.quantize_bf16(plain.float().cpu().numpy() * c)
+    assert (_ulps(want, twice, oracle) != 0).mean() > 0.05
+    with pytest.raises(fv.FvError):
+        fv.qk_norm_rope_bhsd(*args, out_mul=float("nan"))
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_split_and_merge_heads_bit_exact(fv, oracle, dtype):
     import torch

@@ -128,7 +128,8 @@ def test_dense_plan_reaches_the_fused_kernel(fv, oracle, act16, f32_in):
     mk = (lambda x: dev(x)) if f32_in else (lambda x: dev(x).to(torch.bfloat16))
     tq, tk, tv = mk(shape(q, sq)), mk(shape(k, sk)), mk(shape(v, sk))
     before = fv.rt_stats()
-    with fv.with_bf16_act(act16):
+    # (fold off: the reference's order for f32 operands, round then scale; bf16 operands never see the switch)
+    with fv.with_bf16_act(act16), fv.with_fold_scale(False):
         got = fv.sdpa(tq, tk, tv, fv.Plan.dense(None))
     after = fv.rt_stats()
     assert after["fused"] == before["fused"] + 1 and after["composed"] == before["composed"]
@@ -140,6 +141,66 @@ def test_dense_plan_reaches_the_fused_kernel(fv, oracle, act16, f32_in):
     assert torch.equal(got.reshape(b * h, sq, d), direct)
     assert_parity(host(got).reshape(b * h, sq, d), oracle.sdpa_composed(q, k, v), "rt_dense_fused",
                   max_abs=2e-2 if act16 else 1e-2)
+
+
+@pytest.mark.parametrize("kind", ["dense", "dense_scale", "block_causal", "kv_window"])
+def test_f32_queries_take_the_scale_into_their_one_rounding(fv, oracle, kind):
+    """An f32 q is rounded to bf16 by the library itself (rt/sdpa.rs:167-181): with the fold switch on (default) that
+    one rounding is of q * scale * log2(e) and the kernel runs its form for scale = ln 2. Checked: the launch counter
+    of that form moves; the result IS the kernel-level call on bf16(q * c) at ln 2, bit for bit; against the fp32
+    host math on the UNROUNDED q at the plan's scale it is inside the tolerance and as close as the unfolded order
+    (round, then scale) is; bf16 queries give the same bits whatever the switch says."""
+    import torch
+
+    b, h, sq, sk, d = 1, 4, 700, 1100, 128
+    announce(f"rt fold scale into f32 q, {kind}")
+    rng = np.random.Generator(np.random.PCG64(4100))
+    qn = rng.standard_normal((b * h, sq, d), dtype=np.float32)                 # NOT bf16 numbers
+    kn, vn = (oracle.quantize_bf16(rng.standard_normal((b * h, sk, d), dtype=np.float32)) for _ in range(2))
+    if kind in ("block_causal", "kv_window"):
+        sk = sq if kind == "block_causal" else sk
+        kn, vn = kn[:, :sk].copy(), vn[:, :sk].copy()
+    scale = 0.11 if kind == "dense_scale" else None
+    sc = np.float32(scale if scale is not None else 1.0 / np.sqrt(d))
+    bc = fv.BlockCausal(100, 3, 1)
+    plan = {"dense": fv.Plan.dense(None), "dense_scale": fv.Plan.dense(scale), "block_causal": fv.Plan.block_causal(None, bc),
+            "kv_window": fv.Plan.kv_window()}[kind]
+    tq = dev(qn.reshape(b, h, sq, d))
+    tk, tv = (dev(x.reshape(b, h, sk, d)).to(torch.bfloat16) for x in (kn, vn))
+    lib = fv.lib()
+    with fv.with_bf16_act(False):
+        n0 = lib.fv_sdpa_log2_domain_launches()
+        with fv.with_fold_scale(True):
+            folded = fv.sdpa(tq, tk, tv, plan)
+        assert lib.fv_sdpa_log2_domain_launches() == n0 + 1
+        with fv.with_fold_scale(False):
+            plain = fv.sdpa(tq, tk, tv, plan)
+        assert lib.fv_sdpa_log2_domain_launches() == n0 + 1
+        assert fv.fold_scale()                                                # the default is on
+        # bf16 queries: the switch changes nothing
+        q16 = tq.to(torch.bfloat16)
+        with fv.with_fold_scale(True):
+            a = fv.sdpa(q16, tk, tv, plan)
+        with fv.with_fold_scale(False):
+            c = fv.sdpa(q16, tk, tv, plan)
+        assert torch.equal(a, c) and torch.equal(c, plain)                    # ... and is the unfolded f32-q call
+        assert lib.fv_sdpa_log2_domain_launches() == n0 + 1
+    # the kernel-level call the folded route makes
+    cmul = float(np.float32(sc * np.float32(1.4426950408889634)))
+    qc = fv.cast_f32_bf16(tq.reshape(b * h, sq, d), mul=cmul)
+    assert torch.equal(qc, (tq.reshape(b * h, sq, d) * cmul).to(torch.bfloat16))   # one product in f32, one rounding
+    ln2 = float(np.float32(np.log(2.0)))
+    k3, v3 = tk.reshape(b * h, sk, d), tv.reshape(b * h, sk, d)
+    direct = (fv.sdpa_block_causal_bf16(qc, k3, v3, 100, 3, 1, scale=ln2) if kind == "block_causal"
+              else fv.sdpa_dense_bf16(qc, k3, v3, scale=ln2))
+    torch.cuda.synchronize()
+    assert torch.equal(folded.reshape(b * h, sq, d), direct)
+    # against the host math on the f32 q
+    want = oracle.sdpa_composed_rows(qn, kn, vn, np.arange(sq), scale=float(sc),
+                                     mask_bc=(100, 3, 1) if kind == "block_causal" else None)
+    mf = assert_parity(host(folded).reshape(b * h, sq, d), want, f"rt_fold_{kind}", max_rel_l2=1e-2)
+    mp = assert_parity(host(plain).reshape(b * h, sq, d), want, f"rt_unfolded_{kind}", max_rel_l2=1e-2)
+    assert mf["rel_l2"] <= 1.1 * mp["rel_l2"], (mf, mp)
 
 
 def test_backend_setting_steers_the_dense_route(fv, oracle):
