@@ -191,8 +191,9 @@ def test_f32_queries_take_the_scale_into_their_one_rounding(fv, oracle, kind):
     assert torch.equal(qc, (tq.reshape(b * h, sq, d) * cmul).to(torch.bfloat16))   # one product in f32, one rounding
     ln2 = float(np.float32(np.log(2.0)))
     k3, v3 = tk.reshape(b * h, sk, d), tv.reshape(b * h, sk, d)
+    # (dense routes split the keys when the query tiles alone do not fill the GPU: the same choice here)
     direct = (fv.sdpa_block_causal_bf16(qc, k3, v3, 100, 3, 1, scale=ln2) if kind == "block_causal"
-              else fv.sdpa_dense_bf16(qc, k3, v3, scale=ln2))
+              else fv.sdpa_dense_bf16_splitkv(qc, k3, v3, splits=None, scale=ln2))
     torch.cuda.synchronize()
     assert torch.equal(folded.reshape(b * h, sq, d), direct)
     # against the host math on the f32 q
