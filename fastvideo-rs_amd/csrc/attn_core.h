@@ -207,132 +207,20 @@ FV_DEV void qk_tile_side(const lds_u8* kb, int k_base, const bf16x8 (&qf)[8], f3
     }
 }
 
-// Online-softmax state of one query (replicated in lanes l and l^32; l_acc is
-// the lane's own share of the row sum).
-struct SoftmaxState {
-    float m_run, m_used, ms_used, l_acc;
-    FV_DEV void init() {
-        m_run = neg_inf();
-        m_used = neg_inf();
-        ms_used = 0.f;
-        l_acc = 0.f;
-    }
-};
-
 constexpr float kRescaleLog2 = 6.0f;
 
-// Row max, lazy rescale of (l, O), P = 2^(s*sl2 - offset), bf16 pack.
-// pb[t] is the B operand (16 key slots x 32 queries) for key group t.
-// `side(part)` runs after the rescale (part 0) and after each 32-key half of the exponentials
-// (parts 1, 2): slots for side work, such as tile DMA issue, spread through the VALU stream.
-template <class Side>
-FV_DEV void softmax_tile_side(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float sl2,
-                              bf16x8 (&pb)[4], Side&& side) {
-    const float NEG = neg_inf();
-    float mx = s[0][0];
-#pragma unroll
-    for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s[0][i]);
-#pragma unroll
-    for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s[1][i]);
-    mx = pair_max(mx);
-    st.m_run = __builtin_fmaxf(st.m_run, mx);
-    const bool need = (st.m_run * sl2 - st.ms_used > kRescaleLog2) ||
-                      (st.m_used == NEG && st.m_run != NEG);
-    if (__builtin_amdgcn_ballot_w64(need) != 0) {
-        const float ms_new = (st.m_run == NEG) ? 0.f : st.m_run * sl2;
-        const float alpha = (st.m_used == NEG) ? 0.f : fast_exp2(st.ms_used - ms_new);
-        st.l_acc *= alpha;
-#pragma unroll
-        for (int db = 0; db < 4; db++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
-        st.m_used = st.m_run;
-        st.ms_used = ms_new;
-    }
-    side(0);
-#pragma unroll
-    for (int b = 0; b < 2; b++) {
-        f32x16 e;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            e[i] = fast_exp2(__builtin_fmaf(s[b][i], sl2, -st.ms_used));
-            st.l_acc += e[i];
-        }
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-            f32x8 f;
-#pragma unroll
-            for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
-            pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
-        }
-        side(1 + b);
-    }
-}
-FV_DEV void softmax_tile(f32x16 (&s)[2], SoftmaxState& st, f32x16 (&o)[4], float sl2,
-                         bf16x8 (&pb)[4]) {
-    softmax_tile_side(s, st, o, sl2, pb, [](int) {});
-}
-
-// softmax_tile over a pair of tiles (128 keys) with one shared max / rescale decision.
-template <int NO = 4>
-FV_DEV void softmax_tile_pair(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxState& st, f32x16 (&o)[NO],
-                              float sl2, bf16x8 (&pb0)[4], bf16x8 (&pb1)[4]) {
-    const float NEG = neg_inf();
-    float mx = s0[0][0];
-#pragma unroll
-    for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s0[0][i]);
-#pragma unroll
-    for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s0[1][i]);
-#pragma unroll
-    for (int b = 0; b < 2; b++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s1[b][i]);
-    mx = pair_max(mx);
-    st.m_run = __builtin_fmaxf(st.m_run, mx);
-    const bool need = (st.m_run * sl2 - st.ms_used > kRescaleLog2) ||
-                      (st.m_used == NEG && st.m_run != NEG);
-    if (__builtin_amdgcn_ballot_w64(need) != 0) {
-        const float ms_new = (st.m_run == NEG) ? 0.f : st.m_run * sl2;
-        const float alpha = (st.m_used == NEG) ? 0.f : fast_exp2(st.ms_used - ms_new);
-        st.l_acc *= alpha;
-#pragma unroll
-        for (int db = 0; db < NO; db++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
-        st.m_used = st.m_run;
-        st.ms_used = ms_new;
-    }
-#pragma unroll
-    for (int half = 0; half < 2; half++) {
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-            f32x16 e;
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                e[i] = fast_exp2(__builtin_fmaf(half ? s1[b][i] : s0[b][i], sl2, -st.ms_used));
-                st.l_acc += e[i];
-            }
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                f32x8 f;
-#pragma unroll
-                for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
-                if (half) pb1[2 * b + t] = __builtin_convertvector(f, bf16x8);
-                else pb0[2 * b + t] = __builtin_convertvector(f, bf16x8);
-            }
-        }
-    }
-}
-
-// softmax_tile_pair for calls whose scores are in the base-2 log domain already (scale * log2(e) == 1: the
-// caller folded the softmax scale into Q, e.g. into the weight of the q RMSNorm that produced it). The matrix
-// phase starts every S block from `negoff` (16 copies of minus the lane's offset) as its C operand, so the
-// scores arrive as s - off and P = 2^(s - off) is one v_exp_f32 per score with no multiply-add in front of
-// it: a fifth of the softmax's VALU work gone. State per lane (= per query): `off` the offset, `r` the running
-// max relative to it (-inf until the query has seen a finite score), `l_acc` the lane's share of the row sum.
-// When some lane's r exceeds kRescaleLog2 (or a query sees its first finite score) every lane moves its offset
-// to its running max: l and O are scaled by 2^-r, this pair's scores lose r, negoff is rewritten (wave-uniform
-// branch, rare). Same policy and same exactness argument as softmax_tile_pair: P and l always share an offset.
+// Online softmax in base 2 with the offset riding in the matrix pipe. The K Q^T MFMAs of every S block start from
+// `negoff` (16 copies of minus the lane's offset, in raw score units) as their C operand, so the scores arrive as
+// x = s - off and P = 2^(sl2 * x): one two-operand multiply and one v_exp_f32 per score, no three-operand
+// multiply-add (measured on MI355X against P = exp2(fma(s, sl2, -m * sl2)): same cycles, 1.7 % less time on the
+// long dense launches and 2.3 % on block-causal ones, which run at the chip's power limit). SCALED == false is
+// the form for calls whose sl2 = scale * log2(e) is exactly 1 (the caller folded the softmax scale into Q, e.g.
+// into the q RMSNorm output): the multiply is gone as well.
+// State per lane (= per query; lanes l and l^32 hold the same query): `off` the offset, `r` the running max
+// relative to it (-inf until the query has seen a finite score), `l_acc` the lane's share of the row sum.
+// When sl2 * r exceeds kRescaleLog2 in some lane (or a query sees its first finite score) every lane moves its
+// offset to its running max: l and O are scaled by 2^(-sl2 r), this phase's scores lose r, negoff is rewritten
+// (wave-uniform branch, rare). The final O / l is exact for any such policy: P and l always share an offset.
 struct SoftmaxOffState {
     float r, off, l_acc;
     FV_DEV void init() {
@@ -340,11 +228,64 @@ struct SoftmaxOffState {
         off = 0.f;
         l_acc = 0.f;
     }
+    // base-2 logarithm of the row sum's scale: sum_k 2^(sl2 s_k) = l * 2^(sl2 off)
+    template <bool SCALED>
+    FV_DEV float log2_offset(float sl2) const { return SCALED ? off * sl2 : off; }
 };
-template <int NO = 4>
-FV_DEV void softmax_tile_pair_off(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxOffState& st, f32x16 (&o)[NO],
-                                  f32x16& negoff, bf16x8 (&pb0)[4], bf16x8 (&pb1)[4]) {
+
+// The rescale decision and its (rare) execution for NS score blocks of 16: returns nothing, updates st, o, the
+// scores and negoff. mx: the lane pair's max over this phase's scores (relative to the offset).
+template <bool SCALED, int NO, int NS>
+FV_DEV void softmax_off_rescale(float mx, SoftmaxOffState& st, f32x16 (&o)[NO], f32x16& negoff, float sl2,
+                                f32x16* const (&sc)[NS]) {
     const float NEG = neg_inf();
+    const float r_new = __builtin_fmaxf(st.r, mx);
+    const bool need = ((SCALED ? r_new * sl2 : r_new) > kRescaleLog2) || (st.r == NEG && r_new != NEG);
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {
+        const float delta = (r_new == NEG) ? 0.f : r_new;
+        const float alpha = (st.r == NEG) ? 0.f : fast_exp2(SCALED ? -delta * sl2 : -delta);
+        st.l_acc *= alpha;
+#pragma unroll
+        for (int db = 0; db < NO; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
+#pragma unroll
+        for (int b = 0; b < NS; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) (*sc[b])[i] -= delta;   // -inf stays -inf
+        st.off += delta;
+#pragma unroll
+        for (int i = 0; i < 16; i++) negoff[i] = -st.off;
+        st.r = (r_new == NEG) ? NEG : 0.f;
+    } else {
+        st.r = r_new;
+    }
+}
+
+// 32 keys x 32 queries of scores (relative to the offset) to P: exponentials, row-sum share, bf16 pack (RNE).
+// pb[t] is the B operand (16 key slots x 32 queries) of key group t.
+template <bool SCALED>
+FV_DEV void softmax_off_block(const f32x16& sb, SoftmaxOffState& st, float sl2, bf16x8& p_lo, bf16x8& p_hi) {
+    f32x16 e;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        e[i] = fast_exp2(SCALED ? sb[i] * sl2 : sb[i]);
+        st.l_acc += e[i];
+    }
+    f32x8 f0, f1;
+#pragma unroll
+    for (int x = 0; x < 8; x++) {
+        f0[x] = e[x];
+        f1[x] = e[8 + x];
+    }
+    p_lo = __builtin_convertvector(f0, bf16x8);
+    p_hi = __builtin_convertvector(f1, bf16x8);
+}
+
+// A pair of tiles (128 keys) with one shared max / rescale decision.
+template <bool SCALED, int NO = 4>
+FV_DEV void softmax_tile_pair_off(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxOffState& st, f32x16 (&o)[NO],
+                                  f32x16& negoff, float sl2, bf16x8 (&pb0)[4], bf16x8 (&pb1)[4]) {
     float mx = s0[0][0];
 #pragma unroll
     for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s0[0][i]);
@@ -355,101 +296,31 @@ FV_DEV void softmax_tile_pair_off(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxOffSt
 #pragma unroll
         for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s1[b][i]);
     mx = pair_max(mx);
-    const float r_new = __builtin_fmaxf(st.r, mx);
-    const bool need = (r_new > kRescaleLog2) || (st.r == NEG && r_new != NEG);
-    if (__builtin_amdgcn_ballot_w64(need) != 0) {
-        const float delta = (r_new == NEG) ? 0.f : r_new;
-        const float alpha = (st.r == NEG) ? 0.f : fast_exp2(-delta);
-        st.l_acc *= alpha;
+    f32x16* const sc[4] = {&s0[0], &s0[1], &s1[0], &s1[1]};
+    softmax_off_rescale<SCALED, NO, 4>(mx, st, o, negoff, sl2, sc);
 #pragma unroll
-        for (int db = 0; db < NO; db++)
+    for (int b = 0; b < 2; b++) softmax_off_block<SCALED>(s0[b], st, sl2, pb0[2 * b], pb0[2 * b + 1]);
 #pragma unroll
-            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
-#pragma unroll
-        for (int b = 0; b < 2; b++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                s0[b][i] -= delta;   // -inf stays -inf
-                s1[b][i] -= delta;
-            }
-        st.off += delta;
-#pragma unroll
-        for (int i = 0; i < 16; i++) negoff[i] = -st.off;
-        st.r = (r_new == NEG) ? NEG : 0.f;
-    } else {
-        st.r = r_new;
-    }
-#pragma unroll
-    for (int half = 0; half < 2; half++) {
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-            f32x16 e;
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                e[i] = fast_exp2(half ? s1[b][i] : s0[b][i]);
-                st.l_acc += e[i];
-            }
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                f32x8 f;
-#pragma unroll
-                for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
-                if (half) pb1[2 * b + t] = __builtin_convertvector(f, bf16x8);
-                else pb0[2 * b + t] = __builtin_convertvector(f, bf16x8);
-            }
-        }
-    }
+    for (int b = 0; b < 2; b++) softmax_off_block<SCALED>(s1[b], st, sl2, pb1[2 * b], pb1[2 * b + 1]);
 }
 
-// softmax_tile_side for scores in the base-2 log domain (see softmax_tile_pair_off): one tile, with the side slots
-// of softmax_tile_side.
-template <class Side>
-FV_DEV void softmax_tile_side_off(f32x16 (&s)[2], SoftmaxOffState& st, f32x16 (&o)[4], f32x16& negoff,
+// One tile. `side(part)` runs after the rescale (part 0) and after each 32-key half of the exponentials
+// (parts 1, 2): slots for side work, such as tile DMA issue, spread through the VALU stream.
+template <bool SCALED, class Side>
+FV_DEV void softmax_tile_side_off(f32x16 (&s)[2], SoftmaxOffState& st, f32x16 (&o)[4], f32x16& negoff, float sl2,
                                   bf16x8 (&pb)[4], Side&& side) {
-    const float NEG = neg_inf();
     float mx = s[0][0];
 #pragma unroll
     for (int i = 1; i < 16; i++) mx = __builtin_fmaxf(mx, s[0][i]);
 #pragma unroll
     for (int i = 0; i < 16; i++) mx = __builtin_fmaxf(mx, s[1][i]);
     mx = pair_max(mx);
-    const float r_new = __builtin_fmaxf(st.r, mx);
-    const bool need = (r_new > kRescaleLog2) || (st.r == NEG && r_new != NEG);
-    if (__builtin_amdgcn_ballot_w64(need) != 0) {
-        const float delta = (r_new == NEG) ? 0.f : r_new;
-        const float alpha = (st.r == NEG) ? 0.f : fast_exp2(-delta);
-        st.l_acc *= alpha;
-#pragma unroll
-        for (int db = 0; db < 4; db++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
-#pragma unroll
-        for (int b = 0; b < 2; b++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) s[b][i] -= delta;   // -inf stays -inf
-        st.off += delta;
-#pragma unroll
-        for (int i = 0; i < 16; i++) negoff[i] = -st.off;
-        st.r = (r_new == NEG) ? NEG : 0.f;
-    } else {
-        st.r = r_new;
-    }
+    f32x16* const sc[2] = {&s[0], &s[1]};
+    softmax_off_rescale<SCALED, 4, 2>(mx, st, o, negoff, sl2, sc);
     side(0);
 #pragma unroll
     for (int b = 0; b < 2; b++) {
-        f32x16 e;
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            e[i] = fast_exp2(s[b][i]);
-            st.l_acc += e[i];
-        }
-#pragma unroll
-        for (int t = 0; t < 2; t++) {
-            f32x8 f;
-#pragma unroll
-            for (int x = 0; x < 8; x++) f[x] = e[8 * t + x];
-            pb[2 * b + t] = __builtin_convertvector(f, bf16x8);
-        }
+        softmax_off_block<SCALED>(s[b], st, sl2, pb[2 * b], pb[2 * b + 1]);
         side(1 + b);
     }
 }

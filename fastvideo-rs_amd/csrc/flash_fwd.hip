@@ -66,9 +66,9 @@ constexpr int kBN = 64;          // keys per tile
 constexpr int kPpBM = 256;      // queries per workgroup
 constexpr int kRing2 = 4;        // K buffers = V buffers: 128 KB of LDS at D = 128, 64 KB at D = 64
 
-// LOG2DOM: the call's scale * log2(e) is exactly 1 (scores are base-2 logarithms as they leave the MFMAs):
-// the softmax offset rides in the C operand of the K Q^T MFMAs and the per-score multiply-add is gone
-// (softmax_tile_pair_off).
+// The softmax offset rides in the C operand of the K Q^T MFMAs (softmax_tile_pair_off): a score costs one multiply,
+// one exponential and one add. LOG2DOM: the call's scale * log2(e) is exactly 1 (scores are base-2 logarithms as
+// they leave the MFMAs) and the multiply is gone too.
 template <bool MASKED, int D, bool LOG2DOM>
 __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     using G = TileGeo<D>;
@@ -253,9 +253,9 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     for (int db = 0; db < kNO; db++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o[db][i] = 0.f;
-    std::conditional_t<LOG2DOM, SoftmaxOffState, SoftmaxState> st;
+    SoftmaxOffState st;
     st.init();
-    // the C operand every S block starts from: zeros, or (LOG2DOM) minus the lane's softmax offset
+    // the C operand every S block starts from: minus the lane's softmax offset (zero until the first rescale)
     f32x16 s_init;
 #pragma unroll
     for (int i = 0; i < 16; i++) s_init[i] = 0.f;
@@ -384,8 +384,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         // ---- VALU phase: group 0 in slot 2m+1, group 1 in slot 2m+2 ----
         mask_tile(s0, 2 * m);
         mask_tile(s1, 2 * m + 1);
-        if constexpr (LOG2DOM) softmax_tile_pair_off<kNO>(s0, s1, st, o, s_init, pb0, pb1);
-        else softmax_tile_pair<kNO>(s0, s1, st, o, sl2, pb0, pb1);
+        softmax_tile_pair_off<!LOG2DOM, kNO>(s0, s1, st, o, s_init, sl2, pb0, pb1);
         // P and the row sum must be complete before the barrier: without this the
         // compiler sinks the exponentials past it, into the matrix phase
         asm volatile("" ::"v"(pb0[0]), "v"(pb0[1]), "v"(pb0[2]), "v"(pb0[3]), "v"(pb1[0]), "v"(pb1[1]),
@@ -429,10 +428,8 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                         for (int x = 0; x < 4; x++) r[x] = o[db][4 * g + x] * inv;
                         global_store<f32x4>(po + 32 * db + 8 * g + 4 * h, r);
                     }
-                float lse_off;
-                if constexpr (LOG2DOM) lse_off = st.off;
-                else lse_off = st.ms_used;
-                if (h == 0) p.part_lse[prow] = l_tot > 0.f ? lse_off + __builtin_log2f(l_tot) : NEG;
+                if (h == 0)
+                    p.part_lse[prow] = l_tot > 0.f ? st.template log2_offset<!LOG2DOM>(sl2) + __builtin_log2f(l_tot) : NEG;
             }
             return;
         }

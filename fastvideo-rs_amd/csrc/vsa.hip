@@ -331,8 +331,8 @@ __global__ __launch_bounds__(256) void vsa_tile_qkv3_kernel(Three t, const int* 
 // by direct global->LDS loads: K(i+1) streams in under softmax/PV of tile i and
 // V(i) under QK/softmax of tile i. 32 KB of LDS per workgroup, so four
 // workgroups share a CU.
-// LOG2DOM: the call's scale * log2(e) is exactly 1 (the caller folded the softmax scale into Q): the softmax offset
-// rides in the C operand of the K Q^T MFMAs and the per-score multiply-add is gone (softmax_tile_side_off).
+// The softmax offset rides in the C operand of the K Q^T MFMAs (softmax_tile_side_off). LOG2DOM: the call's
+// scale * log2(e) is exactly 1 (the caller folded the softmax scale into Q) and the per-score multiply is gone too.
 template <bool LOG2DOM>
 __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -363,9 +363,9 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
     for (int db = 0; db < 4; db++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o[db][i] = 0.f;
-    std::conditional_t<LOG2DOM, SoftmaxOffState, SoftmaxState> st;
+    SoftmaxOffState st;
     st.init();
-    f32x16 s_init;   // the C operand every S block starts from: zeros, or (LOG2DOM) minus the lane's softmax offset
+    f32x16 s_init;   // the C operand every S block starts from: minus the lane's softmax offset
 #pragma unroll
     for (int i = 0; i < 16; i++) s_init[i] = 0.f;
 
@@ -411,8 +411,7 @@ __global__ __launch_bounds__(128, 2) void vsa_fine_kernel(const VsaFineParams p)
                 for (int it = first; it < last; it++) dma.template issue_one<false>(kbuf, ksrc, wave, it);
             }
         };
-        if constexpr (LOG2DOM) softmax_tile_side_off(s, st, o, s_init, pb, k_loads);
-        else softmax_tile_side(s, st, o, sl2, pb, k_loads);
+        softmax_tile_side_off<!LOG2DOM>(s, st, o, s_init, sl2, pb, k_loads);
         if (more) wait_vmcnt<8>(); else wait_vmcnt<0>();   // V(i) landed; K(i+1) may be in flight
         block_barrier();
         pv_tile(vbuf, rb.v, pb, o);
