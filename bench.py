@@ -8,8 +8,8 @@ crates/fastvideo-gpucheck/src/kernels_attn.rs:368), the MFMA roofline of the
 flash kernel from HIP-event timings, and the CPU baseline (the fp32 host-math
 oracle timed on a bounded sample of query rows, extrapolated to the full call).
 
-Other workloads (--workload cross|causal|causal3|c5|c5cross|tiny|self_d64|vdn32|vsa624|vsa512|prep|kvcache|kvcache1|
-composed|softmax) are for the design notes; the driver's line is the default `self`.
+Other workloads (--workload cross|causal|causal3|c5|c5cross|tiny|self_d64|vdn32|vsa624|vsa512|prep|layer|kvcache|
+kvcache1|composed|softmax) are for the design notes; the driver's line is the default `self`.
 """
 import argparse
 import json
@@ -348,6 +348,82 @@ def bench_prep(args):
     print(json.dumps(rec), flush=True)
 
 
+def bench_layer(args):
+    """One attention layer's device work at the headline shape, producer to consumer: q and k RMSNorm + RoPE
+    (bf16 kernel) and the V split out of a fused bf16 QKV projection [1, 32760, 3*1536], the dense SDPA call,
+    merge_heads of its output; timed both ways: the softmax scale applied by the SDPA kernel (scale 1/sqrt(d)),
+    and folded into q by the producer (out_mul = scale * log2(e), one float) with the SDPA call at ln 2.
+    FLOPs credited are the SDPA call's; the two outputs are compared with each other."""
+    import torch
+
+    import fv_sdpa
+
+    lib = fv_sdpa.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    batch, seq, heads, d = 1, 32760, 12, 128
+    width = heads * d
+    g = torch.Generator(device=dev).manual_seed(20243)
+    proj = torch.randn((batch, seq, 3 * width), generator=g, device=dev).to(torch.bfloat16)
+    w = (1.0 + 0.1 * torch.randn(width, generator=g, device=dev)).float()
+    ang = torch.rand((seq, d // 2), generator=g, device=dev) * 6.0 - 3.0
+    cos = torch.cos(ang).repeat_interleave(2, dim=1).contiguous()
+    sin = torch.sin(ang).repeat_interleave(2, dim=1).contiguous()
+    scale = 1.0 / math.sqrt(d)
+    ln2 = 0.6931471805599453
+    c = scale * 1.4426950408889634
+    flops = 4.0 * heads * seq * seq * d
+
+    def layer(fold):
+        q = fv_sdpa.qk_norm_rope_bhsd(proj, 0, heads, w, (cos, sin), out_mul=c if fold else 1.0)
+        k = fv_sdpa.qk_norm_rope_bhsd(proj, width, heads, w, (cos, sin))
+        v = fv_sdpa.split_heads_bhsd(proj, 2 * width, heads, d)
+        o = fv_sdpa.sdpa_dense_bf16(q.reshape(heads, seq, d), k.reshape(heads, seq, d), v.reshape(heads, seq, d),
+                                    scale=ln2 if fold else scale, out_bf16=True)
+        return fv_sdpa.merge_heads(o.reshape(batch, heads, seq, d))
+
+    def timed(fold):
+        for _ in range(args.warmup):
+            layer(fold)
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for a, b in evs:
+            a.record()
+            layer(fold)
+            b.record()
+        torch.cuda.synchronize()
+        ms = [a.elapsed_time(b) for a, b in evs]
+        return sum(ms) / len(ms)
+
+    res = {}
+    n0 = lib.fv_sdpa_log2_domain_launches()
+    # interleaved, twice each: the clock of the machine drifts by more than the difference looked for
+    runs = {False: [], True: []}
+    for _ in range(2):
+        for fold in (False, True):
+            runs[fold].append(timed(fold))
+    folded_launches = lib.fv_sdpa_log2_domain_launches() - n0
+    assert folded_launches == 2 * (args.warmup + args.steps), folded_launches
+    a, b = layer(False).float(), layer(True).float()
+    torch.cuda.synchronize()
+    diff = (a - b).abs().max().item()
+    cos_ab = float((a.flatten().double() @ b.flatten().double()) / (a.double().norm() * b.double().norm()))
+    for fold in (False, True):
+        ms = sum(runs[fold]) / len(runs[fold])
+        res["scale folded into q by the producer" if fold else "scale applied in the SDPA kernel"] = {
+            "ms_per_layer": round(ms, 4), "runs_ms": [round(x, 4) for x in runs[fold]],
+            "sdpa_tflops_over_layer_time": round(flops / (ms * 1e-3) / 1e12, 1)}
+    ms = sum(runs[True]) / len(runs[True])
+    rec = {
+        "metric": "attention layer (q/k norm+rope, v split, SDPA, merge) ms, Wan-1.3B 480p, bf16", "value": round(ms, 4),
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "fused QKV projection [1,32760,4608] bf16 -> q/k/v BHSD -> dense SDPA H=12 S=32760 d=128 -> merge_heads"},
+        "forms": res, "max_abs_between_forms": diff, "cosine_between_forms": cos_ab,
+    }
+    print(json.dumps(rec), flush=True)
+
+
 def bench_softmax(args):
     """Row softmax entry on score matrices of the shapes the reference materialises: VSA coarse scores
     (12 x 624 rows of 624), a 4096-key chunk, rows of a whole 32760-key call."""
@@ -466,7 +542,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=8,
                     help="untimed launches first; the shader clock under this kernel takes about six launches to settle")
-    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "kvcache", "kvcache1", "composed", "softmax"])
+    ap.add_argument("--workload", default="self", choices=sorted(WORKLOADS) + sorted(VSA_WORKLOADS) + ["prep", "layer", "kvcache", "kvcache1", "composed", "softmax"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline sample budget; 0 skips it")
     ap.add_argument("--out-bf16", type=int, default=1)
     ap.add_argument("--inputs", default="randn", choices=["randn", "zeros"],
@@ -500,6 +576,9 @@ def main():
         return
     if args.workload in ("kvcache", "kvcache1"):
         bench_kvcache(args, 3 if args.workload == "kvcache" else 1)
+        return
+    if args.workload == "layer":
+        bench_layer(args)
         return
     if args.workload == "composed":
         bench_composed(args)

@@ -304,6 +304,18 @@ FV_DEV void softmax_tile_pair_off(f32x16 (&s0)[2], f32x16 (&s1)[2], SoftmaxOffSt
     for (int b = 0; b < 2; b++) softmax_off_block<SCALED>(s1[b], st, sl2, pb1[2 * b], pb1[2 * b + 1]);
 }
 
+// A pair of tiles with the offset left where it is: no row max, no rescale decision. For walks whose caller
+// checks afterwards that no row sum outgrew the f32 range comfortably (and redoes the walk with
+// softmax_tile_pair_off if one did).
+template <bool SCALED>
+FV_DEV void softmax_tile_pair_fixed(const f32x16 (&s0)[2], const f32x16 (&s1)[2], SoftmaxOffState& st, float sl2,
+                                    bf16x8 (&pb0)[4], bf16x8 (&pb1)[4]) {
+#pragma unroll
+    for (int b = 0; b < 2; b++) softmax_off_block<SCALED>(s0[b], st, sl2, pb0[2 * b], pb0[2 * b + 1]);
+#pragma unroll
+    for (int b = 0; b < 2; b++) softmax_off_block<SCALED>(s1[b], st, sl2, pb1[2 * b], pb1[2 * b + 1]);
+}
+
 // One tile. `side(part)` runs after the rescale (part 0) and after each 32-key half of the exponentials
 // (parts 1, 2): slots for side work, such as tile DMA issue, spread through the VALU stream.
 template <bool SCALED, class Side>

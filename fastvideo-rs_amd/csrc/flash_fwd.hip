@@ -57,6 +57,9 @@
 // positions: a masked call walks up to three ascending tile ranges (block-causal:
 // sink tiles, then the band; VDN window: rows before the video + frame 0, the
 // window frames, the last frame + rows after the video).
+#include <stdlib.h>
+#include <string.h>
+
 #include "attn_core.h"
 #include "fv_internal.h"
 
@@ -65,20 +68,33 @@ namespace fv {
 constexpr int kBN = 64;          // keys per tile
 constexpr int kPpBM = 256;      // queries per workgroup
 constexpr int kRing2 = 4;        // K buffers = V buffers: 128 KB of LDS at D = 128, 64 KB at D = 64
+constexpr int kVoteBytes = 64;   // behind the rings: one word per wave for the fixed-offset pass's vote
 
-// The softmax offset rides in the C operand of the K Q^T MFMAs (softmax_tile_pair_off): a score costs one multiply,
-// one exponential and one add. LOG2DOM: the call's scale * log2(e) is exactly 1 (scores are base-2 logarithms as
-// they leave the MFMAs) and the multiply is gone too.
-template <bool MASKED, int D, bool LOG2DOM>
-__global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
+// Workgroups that had to redo their pass with the running max (see flash_item) since the library was loaded on
+// this device.
+__device__ unsigned long long g_exact_pass_reruns;
+
+// One workgroup's item: the whole pass over its key tiles and the store of its rows. Returns false (FIXED only,
+// nothing stored) when the pass has to be made again with the running max.
+// FIXED: once the first phase has put every query's offset at the largest score of its first 128 keys, the offset
+// stays there: no row max and no rescale decision in the loop (32 three-operand VALU instructions a phase less:
+// 2 % of the time of the long launches, 9 % at head dim 64). Exact for any input as long as nothing overflows (P
+// and l share the offset), so the pass is checked before anything is stored: if some row's scores grew by more
+// than about 2^60 past that first maximum (a row sum outside the comfortable f32 range, or an accumulator not
+// finite), the workgroup makes the pass again from the top with the running max. One difference in rounding
+// remains: the largest P of a row is exactly 1 under the running max and a rounded bf16 number under the fixed
+// offset, so a row that ONE late key dominates can be off by up to 2^-8 relative; the launcher therefore takes
+// this form only for results that are rounded to bf16 anyway.
+template <bool MASKED, int D, bool LOG2DOM, bool FIXED, class Params>
+FV_DEV bool flash_item(const Params& p, const int wave, const int lane, const int block) {
+    static_assert(!(MASKED && FIXED), "a masked query may see none of its first 128 keys: the running max stays");
     using G = TileGeo<D>;
     constexpr int kD = D;
     constexpr int kTileBytes = G::kTile;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     lds_u8* smem = (lds_u8*)smem_raw;
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: branches on it stay scalar
+    const int tid = wave * 64 + lane;   // (wave is scalar: branches on it stay scalar)
     const int grp = wave >> 2;
     const int h = lane >> 5, c32 = lane & 31;
     // Work order. Dense (equal tiles): workgroup i runs on XCD i % 8, and XCD x takes the
@@ -89,15 +105,15 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     // first); measured 9 % faster than the dense order, whose per-XCD ranges hold unequal work.
     int bh, qt, sp = 0;   // sp: this workgroup's key split (dense launches with kv_split > 1)
     if constexpr (MASKED) {
-        const int work = blockIdx.x;
-        if (work >= p.total) return;
+        const int work = block;
+        if (work >= p.total) return true;
         const int nbh = p.total / p.nqt;
         bh = work % nbh;
         const int r = work / nbh;
         qt = p.mask_mode == 2 ? ((r & 1) ? (r >> 1) : p.nqt - 1 - (r >> 1)) : p.nqt - 1 - r;
     } else {
-        const int work = (blockIdx.x & 7) * p.per_xcd + (blockIdx.x >> 3);
-        if (work >= p.total) return;
+        const int work = (block & 7) * p.per_xcd + (block >> 3);
+        if (work >= p.total) return true;
         const int per_bh = p.nqt * p.kv_split;
         bh = work / per_bh;
         const int rem = work - bh * per_bh;
@@ -173,7 +189,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                                    : (char*)(out_f32 + ((size_t)bh * sq + q0) * kD);
             const u32x4 zero = {0u, 0u, 0u, 0u};
             for (int u = tid; u < qlen * units; u += 512) global_store<u32x4>(ob + (size_t)u * 16, zero);
-            return;
+            return true;
         }
     }
     const int np = (ne + 1) / 2;             // phases
@@ -384,7 +400,8 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
         // ---- VALU phase: group 0 in slot 2m+1, group 1 in slot 2m+2 ----
         mask_tile(s0, 2 * m);
         mask_tile(s1, 2 * m + 1);
-        softmax_tile_pair_off<!LOG2DOM, kNO>(s0, s1, st, o, s_init, sl2, pb0, pb1);
+        if (FIXED && !first) softmax_tile_pair_fixed<!LOG2DOM>(s0, s1, st, sl2, pb0, pb1);
+        else softmax_tile_pair_off<!LOG2DOM, kNO>(s0, s1, st, o, s_init, sl2, pb0, pb1);
         // P and the row sum must be complete before the barrier: without this the
         // compiler sinks the exponentials past it, into the matrix phase
         asm volatile("" ::"v"(pb0[0]), "v"(pb0[1]), "v"(pb0[2]), "v"(pb0[3]), "v"(pb1[0]), "v"(pb1[1]),
@@ -410,6 +427,28 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
     pv_tile<D>(vbuf(2 * np - 2), rb.v, pb0, o);
     pv_tile<D>(vbuf(2 * np - 1), rb.v, pb1, o);
 
+    if constexpr (FIXED) {
+        // Did the fixed offset hold? Every row sum comfortably inside the f32 range and every accumulator finite
+        // (x * 0 is NaN for an infinite or NaN x). One vote per wave through 8 words of LDS behind the rings.
+        float chk = 0.f;
+#pragma unroll
+        for (int db = 0; db < kNO; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) chk = __builtin_fmaf(o[db][i], 0.f, chk);
+        const bool lane_ok = (pair_sum(st.l_acc) < 0x1p+64f) && (chk == 0.f);
+        auto* votes = (__attribute__((address_space(3))) unsigned*)(smem + 2 * kRing2 * kTileBytes);
+        if (lane == 0) votes[wave] = __builtin_amdgcn_ballot_w64(!lane_ok) != 0 ? 1u : 0u;
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the vote is written before the barrier
+        block_barrier();   // ... behind which every wave is past its last read of both rings
+        const u32x4 v0 = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(votes);
+        const u32x4 v1 = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(votes + 4);
+        const unsigned any = v0[0] | v0[1] | v0[2] | v0[3] | v1[0] | v1[1] | v1[2] | v1[3];
+        if (__builtin_amdgcn_readfirstlane(any) != 0) {
+            if (tid == 0) atomicAdd(&g_exact_pass_reruns, 1ull);
+            return false;
+        }
+    }
+
     const float l_tot = pair_sum(st.l_acc);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int row = wave * 32 + c32;
@@ -431,7 +470,7 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                 if (h == 0)
                     p.part_lse[prow] = l_tot > 0.f ? st.template log2_offset<!LOG2DOM>(sl2) + __builtin_log2f(l_tot) : NEG;
             }
-            return;
+            return true;
         }
     }
     if (out_is_bf16) {
@@ -479,6 +518,31 @@ __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
                     global_store<f32x4>(out_f32 + base + d0, r);
                 }
             }
+    }
+    return true;
+}
+
+// The softmax offset rides in the C operand of the K Q^T MFMAs (softmax_tile_pair_off): a score costs one multiply,
+// one exponential and one add. LOG2DOM: the call's scale * log2(e) is exactly 1 (scores are base-2 logarithms as
+// they leave the MFMAs) and the multiply is gone too. FIXED (dense launches that write bf16): the first pass keeps
+// the offset of the first 128 keys (flash_item); the others keep the running max throughout.
+template <bool MASKED, int D, bool LOG2DOM, bool FIXED>
+__global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {
+    const int tid = threadIdx.x;
+    int wave = __builtin_amdgcn_readfirstlane(tid >> 6), block = blockIdx.x;
+    if constexpr (!FIXED) {
+        flash_item<MASKED, D, LOG2DOM, false>(p, wave, tid & 63, block);
+    } else {
+        if (flash_item<MASKED, D, LOG2DOM, true>(p, wave, tid & 63, block)) return;
+        // The second pass shares nothing with the first but two scalars: its inputs are made opaque (the lane
+        // index counted anew from the execution mask, the kernel arguments read again from their segment, of which
+        // FlashParams is the whole), so that the compiler keeps no value of the first pass alive for it. It runs
+        // once in a blue moon; the first pass is the kernel.
+        using ConstParams = const __attribute__((address_space(4))) FlashParams;
+        ConstParams* again = (ConstParams*)__builtin_amdgcn_kernarg_segment_ptr();
+        int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        asm volatile("" : "+v"(lane), "+s"(wave), "+s"(block), "+s"(again));
+        flash_item<MASKED, D, LOG2DOM, false>(*again, wave, lane, block);
     }
 }
 
@@ -538,42 +602,68 @@ extern "C" int fv_internal_flash_block_m(void) { return fv::kPpBM; }
 
 namespace {
 // The kernel's dynamic LDS limit (128 KB at D = 128), once per device.
-template <bool MASKED, int D, bool LOG2DOM>
+template <bool MASKED, int D, bool LOG2DOM, bool FIXED>
 hipError_t flash_attr() {
     static std::atomic<unsigned long long> attr_done;
-    constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
-    return fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<MASKED, D, LOG2DOM>, lds, attr_done);
+    constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile + fv::kVoteBytes;
+    return fv_set_max_lds_once((const void*)fv::flash_fwd_pp2<MASKED, D, LOG2DOM, FIXED>, lds, attr_done);
 }
-template <bool MASKED, int D, bool LOG2DOM>
+template <bool MASKED, int D, bool LOG2DOM, bool FIXED>
 hipError_t launch_flash_as(const fv::FlashParams* p, hipStream_t stream) {
-    constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile;
-    hipError_t e = flash_attr<MASKED, D, LOG2DOM>();
+    constexpr int lds = 2 * fv::kRing2 * fv::TileGeo<D>::kTile + fv::kVoteBytes;
+    hipError_t e = flash_attr<MASKED, D, LOG2DOM, FIXED>();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((fv::flash_fwd_pp2<MASKED, D, LOG2DOM>), dim3(p->per_xcd * 8), dim3(512), lds, stream, *p);
+    hipLaunchKernelGGL((fv::flash_fwd_pp2<MASKED, D, LOG2DOM, FIXED>), dim3(p->per_xcd * 8), dim3(512), lds, stream, *p);
     return hipGetLastError();
 }
+// FASTVIDEO_SDPA_RUNNING_MAX=1: every launch keeps the running max (no fixed-offset first pass).
+bool running_max_forced() {
+    static const bool v = [] {
+        const char* e = getenv("FASTVIDEO_SDPA_RUNNING_MAX");
+        return e && *e && strcmp(e, "0") != 0;
+    }();
+    return v;
+}
 // A call whose scale * log2(e) is exactly 1 (scale = ln 2: the caller folded the softmax scale into Q) runs
-// the form without the per-score multiply-add.
+// the form without the per-score multiply.
 std::atomic<unsigned long long> g_log2_domain_launches{0};
+template <bool MASKED, int D, bool FIXED>
+hipError_t launch_flash_fixed(const fv::FlashParams* p, hipStream_t stream) {
+    if (p->sl2 != 1.0f) return launch_flash_as<MASKED, D, false, FIXED>(p, stream);
+    g_log2_domain_launches.fetch_add(1, std::memory_order_relaxed);
+    return launch_flash_as<MASKED, D, true, FIXED>(p, stream);
+}
+// Dense launches whose result is rounded to bf16 make their first pass with the fixed offset: on a row that one
+// late key dominates, that key's P is then a rounded bf16 number instead of exactly 1 (up to 2^-8 relative on the
+// row), which a bf16 result absorbs; f32 results and masked launches keep the running max.
 template <bool MASKED, int D>
 hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
-    if (p->sl2 != 1.0f) return launch_flash_as<MASKED, D, false>(p, stream);
-    g_log2_domain_launches.fetch_add(1, std::memory_order_relaxed);
-    return launch_flash_as<MASKED, D, true>(p, stream);
+    if constexpr (!MASKED) {
+        if (p->out_is_bf16 && !running_max_forced()) return launch_flash_fixed<MASKED, D, true>(p, stream);
+    }
+    return launch_flash_fixed<MASKED, D, false>(p, stream);
 }
 }  // namespace
 
 extern "C" uint64_t fv_sdpa_log2_domain_launches(void) { return g_log2_domain_launches.load(std::memory_order_relaxed); }
 
+extern "C" hipError_t fv_internal_exact_pass_reruns(unsigned long long* out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(fv::g_exact_pass_reruns), sizeof *out, 0, hipMemcpyDeviceToHost);
+}
+
 extern "C" hipError_t fv_internal_init_flash(void) {
-    hipError_t e = flash_attr<false, 128, false>();
-    if (e == hipSuccess) e = flash_attr<true, 128, false>();
-    if (e == hipSuccess) e = flash_attr<false, 64, false>();
-    if (e == hipSuccess) e = flash_attr<true, 64, false>();
-    if (e == hipSuccess) e = flash_attr<false, 128, true>();
-    if (e == hipSuccess) e = flash_attr<true, 128, true>();
-    if (e == hipSuccess) e = flash_attr<false, 64, true>();
-    if (e == hipSuccess) e = flash_attr<true, 64, true>();
+    hipError_t e = flash_attr<false, 128, false, false>();
+    if (e == hipSuccess) e = flash_attr<true, 128, false, false>();
+    if (e == hipSuccess) e = flash_attr<false, 64, false, false>();
+    if (e == hipSuccess) e = flash_attr<true, 64, false, false>();
+    if (e == hipSuccess) e = flash_attr<false, 128, true, false>();
+    if (e == hipSuccess) e = flash_attr<true, 128, true, false>();
+    if (e == hipSuccess) e = flash_attr<false, 64, true, false>();
+    if (e == hipSuccess) e = flash_attr<true, 64, true, false>();
+    if (e == hipSuccess) e = flash_attr<false, 128, false, true>();
+    if (e == hipSuccess) e = flash_attr<false, 64, false, true>();
+    if (e == hipSuccess) e = flash_attr<false, 128, true, true>();
+    if (e == hipSuccess) e = flash_attr<false, 64, true, true>();
     return e;
 }
 

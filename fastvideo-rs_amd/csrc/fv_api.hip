@@ -213,6 +213,11 @@ int fv_sdpa_init(void) {
 // the launcher's own test (flash_fwd.hip launch_flash): FlashParams::sl2, computed as below, equal to one
 int fv_sdpa_is_log2_domain_scale(float scale) { return scale * 1.4426950408889634f == 1.0f ? 1 : 0; }
 
+uint64_t fv_sdpa_exact_pass_reruns(void) {
+    unsigned long long n = 0;
+    return fv_internal_exact_pass_reruns(&n) == hipSuccess ? (uint64_t)n : 0;
+}
+
 int fv_sdpa_supported(size_t b, size_t h, size_t sq, size_t sk, size_t d) {
     if (b != 0 && h > (size_t)65535 / b) return 0;
     const size_t bh = b * h;

@@ -119,6 +119,7 @@ __host__ __device__ inline TileWalk mask_tile_walk(const FlashParams& p, int q0,
 extern "C" int fv_internal_flash_block_m(void);   // queries per workgroup of the flash kernel in use
 extern "C" hipError_t fv_internal_launch_flash(const fv::FlashParams* p, int masked, int d,
                                                hipStream_t stream);
+extern "C" hipError_t fv_internal_exact_pass_reruns(unsigned long long* out);
 extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16, const int* slot_src,
                                                    const int* block_sizes, float* out, size_t bh,
                                                    size_t seq, int dim, int num_tiles, int round16,

@@ -24,6 +24,7 @@ SIGNATURES = {
     "fv_sdpa_supported": (C.c_int, [_sz, _sz, _sz, _sz, _sz]),
     "fv_sdpa_is_log2_domain_scale": (C.c_int, [C.c_float]),
     "fv_sdpa_log2_domain_launches": (C.c_uint64, []),
+    "fv_sdpa_exact_pass_reruns": (C.c_uint64, []),
     "fv_sdpa_dense_bf16": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float, _vp]),
     "fv_sdpa_dense_bf16_strided": (C.c_int, [_vp, _vp, _vp, _vp, C.c_int, _sz, _sz, _sz, _sz, C.c_float, _sz, _sz, _sz,
                                              _vp]),

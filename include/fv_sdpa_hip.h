@@ -60,6 +60,14 @@ int fv_sdpa_is_log2_domain_scale(float scale);
 /* Launches of that form of the dense / masked kernel since the library was loaded (all its entries together). */
 uint64_t fv_sdpa_log2_domain_launches(void);
 
+/* No counterpart in the reference (a diagnostic). Dense launches make their pass over the keys with every query's
+ * softmax offset fixed at the largest score of its first 128 keys (no running max in the loop), check the row sums
+ * and accumulators before anything is stored, and make the pass again with the running max in any workgroup where
+ * a row's scores outgrew that offset by more than about 2^60: results are exact either way, the second pass only
+ * costs time. This is the number of workgroups that took it on the current device since the library was loaded.
+ * Blocks until the device's work so far is done (a device-to-host copy of the counter); 0 without a device. */
+uint64_t fv_sdpa_exact_pass_reruns(void);
+
 /* rt/attn.rs:283-421 `device_mma_sdpa_with` + kernels/attn2.cu:607-621
  * `flash_mma_fwd2_d128` / `_d64`: out = softmax(scale * q k^T) v.
  * q [bh,sq,128], k/v [bh,sk,128] bf16 bits; out is f32 [bh,sq,128] when

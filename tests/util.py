@@ -73,3 +73,24 @@ def sample_rows(seed, sq, n, extra=()):
     rows = set(int(r) for r in rng.choice(sq, size=min(n, sq), replace=False))
     rows.update(int(r) for r in extra if 0 <= r < sq)
     return np.array(sorted(rows), dtype=np.int64)
+
+
+
+def assert_bf16_result_matches_f32_result(got16, got32, tag, exact_share=0.0):
+    """A launch that writes bf16 against the same launch writing f32. Dense launches that write bf16 keep their softmax
+    offset fixed after the first 128 keys where the f32 ones follow the running max: the same arithmetic, hence the
+    RNE rounding of the f32 result bit for bit, for every wave in which no row's maximum grows by 2^6 after its first
+    128 keys; two roundings of P apart otherwise (each about 1.6e-3 of the result's rms in l2, several times that at
+    the worst of millions of elements). Bar: every element within half a bf16 step of the f32 value plus 4e-2 of the
+    result's rms, and at least `exact_share` of the elements equal to the rounded f32 value."""
+    import oracle
+
+    a = np.asarray(got16, dtype=np.float32)
+    b = np.asarray(got32, dtype=np.float32)
+    rms = float(np.sqrt(np.mean(b.astype(np.float64) ** 2)))
+    excess = np.abs(a - b) - (2.0 ** -8 * np.abs(b) + 4e-2 * rms)
+    share = float(np.mean(a == oracle.quantize_bf16(b)))
+    print(f"[bf16-vs-f32] {tag}: {100 * share:.3f} % of the elements are the rounded f32 value, worst excess {excess.max():.2e}",
+          flush=True)
+    assert excess.max() <= 0, f"{tag}: {excess.max()}"
+    assert share >= exact_share, f"{tag}: only {share} of the elements are the rounded f32 value"
