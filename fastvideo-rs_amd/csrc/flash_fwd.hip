@@ -87,7 +87,7 @@ __device__ unsigned long long g_exact_pass_reruns;
 // this form only for results that are rounded to bf16 anyway.
 template <bool MASKED, int D, bool LOG2DOM, bool FIXED, class Params>
 FV_DEV bool flash_item(const Params& p, const int wave, const int lane, const int block) {
-    static_assert(!(MASKED && FIXED), "a masked query may see none of its first 128 keys: the running max stays");
+    // (masked launches: only where every query sees a key among the walk's first 128, see launch_flash)
     using G = TileGeo<D>;
     constexpr int kD = D;
     constexpr int kTileBytes = G::kTile;
@@ -633,14 +633,16 @@ hipError_t launch_flash_fixed(const fv::FlashParams* p, hipStream_t stream) {
     g_log2_domain_launches.fetch_add(1, std::memory_order_relaxed);
     return launch_flash_as<MASKED, D, true, FIXED>(p, stream);
 }
-// Dense launches whose result is rounded to bf16 make their first pass with the fixed offset: on a row that one
-// late key dominates, that key's P is then a rounded bf16 number instead of exactly 1 (up to 2^-8 relative on the
-// row), which a bf16 result absorbs; f32 results and masked launches keep the running max.
+// Launches whose result is rounded to bf16 make their first pass with the fixed offset: on a row that one late
+// key dominates, that key's P is then a rounded bf16 number instead of exactly 1 (up to 2^-8 relative on the row),
+// which a bf16 result absorbs; f32 results keep the running max. Masked launches take it where every query sees a
+// key among the first 128 of its tile's walk, so that its offset is a score of its own: block-causal without a
+// window (key 0 is visible to every query). Under a window, or the VDN mask, a query's first visible key may lie
+// anywhere in the walk: those keep the running max.
 template <bool MASKED, int D>
 hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
-    if constexpr (!MASKED) {
-        if (p->out_is_bf16 && !running_max_forced()) return launch_flash_fixed<MASKED, D, true>(p, stream);
-    }
+    const bool offset_is_a_score = !MASKED || (p->mask_mode == 1 && p->win == 0);
+    if (p->out_is_bf16 && offset_is_a_score && !running_max_forced()) return launch_flash_fixed<MASKED, D, true>(p, stream);
     return launch_flash_fixed<MASKED, D, false>(p, stream);
 }
 }  // namespace
@@ -664,6 +666,10 @@ extern "C" hipError_t fv_internal_init_flash(void) {
     if (e == hipSuccess) e = flash_attr<false, 64, false, true>();
     if (e == hipSuccess) e = flash_attr<false, 128, true, true>();
     if (e == hipSuccess) e = flash_attr<false, 64, true, true>();
+    if (e == hipSuccess) e = flash_attr<true, 128, false, true>();
+    if (e == hipSuccess) e = flash_attr<true, 64, false, true>();
+    if (e == hipSuccess) e = flash_attr<true, 128, true, true>();
+    if (e == hipSuccess) e = flash_attr<true, 64, true, true>();
     return e;
 }
 

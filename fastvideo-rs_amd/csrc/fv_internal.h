@@ -65,7 +65,9 @@ struct VsaFineParams {
 struct TileWalk {
     int a1, a2, n0, n1, ne;
 };
-__host__ __device__ inline TileWalk mask_tile_walk(const FlashParams& p, int q0, int qlen, int nkt) {
+// (Params: FlashParams, or the same struct read through another address space)
+template <class Params>
+__host__ __device__ inline TileWalk mask_tile_walk(const Params& p, int q0, int qlen, int nkt) {
     constexpr int kKeys = 64;
     const int sk = p.sk;
     auto imin = [](int a, int b) { return a < b ? a : b; };

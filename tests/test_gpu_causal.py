@@ -207,3 +207,45 @@ def test_full_size_prefix_and_block_properties(fv, bt, win, sink):
         torch.cuda.synchronize()
         delta = (first - full[:, :bt]).abs().max().item()
         assert delta <= min(1e-2, 0.25 * first.std().item()), delta
+
+
+@pytest.mark.parametrize("d", [128, 64])
+def test_block_causal_pass_with_the_fixed_offset_and_its_rerun(fv, oracle, d):
+    """Block-causal launches without a window that write bf16 make their pass with every query's softmax offset fixed
+    at the largest score among the first 128 keys of its tile's walk (key 0 is visible to every query) and redo it with
+    the running max where a row outgrew that by more than about 2^60. One head's later keys score hundreds of base-2
+    units above its first ones: its workgroups take the second pass (counted), every row matches the f64 host math
+    under the mask, the other heads' rows are the bits of a launch without that head, and a launch under a window
+    (whose queries may see none of the walk's first keys) keeps the running max: no rerun, same tolerance."""
+    import torch
+
+    bh, s, bt = 3, 700, 100
+    announce(f"block-causal fixed-offset pass and its rerun d={d}")
+    rng = np.random.Generator(np.random.PCG64(515))
+    q = rng.standard_normal((bh, s, d)).astype(np.float32)
+    k = rng.standard_normal((bh, s, d)).astype(np.float32)
+    v = oracle.quantize_bf16(rng.standard_normal((bh, s, d)).astype(np.float32))
+    q[0] = np.abs(q[0]) + 2.0
+    k[0, :128] = -0.5
+    k[0, 128:] = np.linspace(1.0, 30.0, s - 128, dtype=np.float32)[:, None]
+    q, k = oracle.quantize_bf16(q), oracle.quantize_bf16(k)
+    tq, tk, tv = (to_dev_bf16(x) for x in (q, k, v))
+    lib = fv.lib()
+    n0 = lib.fv_sdpa_exact_pass_reruns()
+    got = fv.sdpa_block_causal_bf16(tq, tk, tv, bt, 0, 0, out_bf16=True)
+    torch.cuda.synchronize()
+    n1 = lib.fv_sdpa_exact_pass_reruns()
+    # head 0: the query tiles whose rows see keys past the first 128 (all three: the first tile's rows 128.. do)
+    assert n1 - n0 == (s + 255) // 256, (n0, n1)
+    want = oracle.sdpa_f64(q, k, v, mask_bc=(bt, 0, 0))
+    assert_parity(got.float().cpu().numpy(), want, f"causal_rerun_d{d}", max_abs=2e-2)
+    rest = fv.sdpa_block_causal_bf16(tq[1:].contiguous(), tk[1:].contiguous(), tv[1:].contiguous(), bt, 0, 0, out_bf16=True)
+    torch.cuda.synchronize()
+    assert lib.fv_sdpa_exact_pass_reruns() == n1 and torch.equal(rest, got[1:])
+    # f32 results and windowed masks keep the running max
+    got32 = fv.sdpa_block_causal_bf16(tq, tk, tv, bt, 0, 0)
+    gotw = fv.sdpa_block_causal_bf16(tq, tk, tv, bt, 3, 1, out_bf16=True)
+    torch.cuda.synchronize()
+    assert lib.fv_sdpa_exact_pass_reruns() == n1
+    assert_parity(got32.cpu().numpy(), want, f"causal_running_max_d{d}")
+    assert_parity(gotw.float().cpu().numpy(), oracle.sdpa_f64(q, k, v, mask_bc=(bt, 3, 1)), f"causal_window_d{d}", max_abs=2e-2)
