@@ -27,7 +27,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the flash kernel at the headline workload. NOT measured by this script: the figure
 # comes from two rocprofv3 --pmc runs of this same command (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, the
 # factors from a plain 1 GiB copy in the same runs), whose summary is the file named beside it.
-MEASURED_TRAFFIC_BYTES = {"self": (1.0065e9, "profiles/flash_fwd_pp2_wan13b_self_attention.md")}
+MEASURED_TRAFFIC_BYTES = {"self": (1.0069e9, "profiles/flash_fwd_pp2_wan13b_self_attention.md")}
 
 WORKLOADS = {
     # name: (H, Sq, Sk, causal block_tokens or 0, description)
@@ -220,7 +220,7 @@ def bench_kvcache(args, fpb=3):
         "ms_per_step_with_window_copies_no_split": round(copied, 4), "ms_per_step_in_place_no_split": round(unsplit, 4),
         "ms_per_step_eager_python_loop": round(eager, 4),
         "roofline": {"bound": "mfma", "achieved": round(tf, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::flash_fwd_pp2<false, 128, false>"},
+                     "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": "fv::flash_fwd_pp2<false, 128, false, true>"},
     }
     print(json.dumps(rec), flush=True)
 
@@ -676,7 +676,10 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": f"fv::flash_fwd_pp2<{'true' if bt else 'false'}, {d}, {'true' if args.fold_scale else 'false'}>",
+                     # template arguments: masked, head dim, scale folded into Q, fixed-offset first pass (launches
+                     # that write bf16: dense, and block-causal without a window)
+                     "kernel": f"fv::flash_fwd_pp2<{'true' if bt else 'false'}, {d}, {'true' if args.fold_scale else 'false'}, "
+                               f"{'true' if args.out_bf16 and bt >= 0 else 'false'}>",
                      "avg_kernel_ms": round(avg_kernel_ms, 4), "median_kernel_ms": round(kern_ms[len(kern_ms) // 2], 4),
                      "min_hbm_bytes": bytes_min,
                      "hbm_frac_at_min_traffic": round(bytes_min / (avg_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
