@@ -71,7 +71,12 @@ uint64_t fv_sdpa_exact_pass_reruns(void);
 /* rt/attn.rs:283-421 `device_mma_sdpa_with` + kernels/attn2.cu:607-621
  * `flash_mma_fwd2_d128` / `_d64`: out = softmax(scale * q k^T) v.
  * q [bh,sq,128], k/v [bh,sk,128] bf16 bits; out is f32 [bh,sq,128] when
- * out_is_bf16 == 0, else bf16 bits (RNE). scale > 0. */
+ * out_is_bf16 == 0, else bf16 bits (RNE). scale > 0.
+ * Rounding: with out_is_bf16 == 0 every row follows its running maximum (its largest P is exactly 1); with
+ * out_is_bf16 == 1 the softmax offset of a row is the largest score of its first 128 keys (see
+ * fv_sdpa_exact_pass_reruns), so a row that one later key dominates carries that key's bf16-rounded P: up to 2^-8
+ * relative on such a row, beside the 2^-8 of the result's own rounding. FASTVIDEO_SDPA_RUNNING_MAX=1 (read once)
+ * keeps the running maximum in every launch. */
 int fv_sdpa_dense_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                        int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                        void* stream);
@@ -125,7 +130,10 @@ int fv_sdpa_dense_bf16_splitkv_static(const uint16_t* q, const uint16_t* k, cons
  * `flash_mma_fwd2_causal_d128`: the same under BlockCausal{block_tokens,
  * window, sink} (rt/attn.rs:441-453): query i sees key j iff
  * (tj <= ti && (window == 0 || ti - tj < window)) || tj < sink, t = idx / block_tokens.
- * Key tiles no query of a workgroup can see are never loaded. */
+ * Key tiles no query of a workgroup can see are never loaded. A query that sees no key at all (more queries than
+ * keys under a window that has moved past the last key) gets a row of zeros, what the reference's fused kernel
+ * stores for a row without a visible key (kernels/attn2.cu:150); its composed route with the additive -1e9 mask
+ * (rt/attn.rs:455-467) would give such a row the mean of V. No reference fixture covers the case: parity unpinned. */
 int fv_sdpa_block_causal_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                               int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d,
                               float scale, size_t block_tokens, size_t window, size_t sink,
