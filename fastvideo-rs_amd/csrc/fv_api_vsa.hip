@@ -331,27 +331,22 @@ static int vsa_attention_common(const void* q, const void* k, const void* v, int
     hipStream_t st = (hipStream_t)stream;
     hipError_t e;
     int rc;
-    // 4 (moved up). tile-ordered bf16 copies for the fine stage (rt/vsa.rs:406-414): q, k and v in one launch
-    if (!tiled) {
-        uint16_t* const tiles[3] = {(uint16_t*)(ws + w.qt), (uint16_t*)(ws + w.kt), (uint16_t*)(ws + w.vt)};
-        const void* const src[3] = {q, k, v};
-        if (dim % 8 != 0 || !fits_int(padded * (dim / 8) / 256 + 1)) return fv_decline("vsa_attention: tile pass too large");
-        e = fv_internal_launch_tile_qkv3(src, qkv_is_bf16, slot_src, tiles, bh, seq, padded, (int)dim, st);
-        if (e != hipSuccess) return fv_fail_hip(e, "vsa_tile_qkv");
-        qt = tiles[0], kt = tiles[1], vt = tiles[2];
-    }
-    // 1. tile means (rt/vsa.rs:378-384), one launch. Of bf16 operands they are taken from the tile-ordered
-    //    copies (the same values in the same slot order, read as contiguous rows: half the time of the
-    //    gather from token order); f32 operands are pooled unrounded, so they are read where they lie.
+    // 1 + 4. tile means (rt/vsa.rs:378-384) and the tile-ordered bf16 copies for the fine stage (rt/vsa.rs:406-414)
+    //    of q, k and v in ONE scan: every token row is read once, written to its slot as bf16 and added, unrounded
+    //    and in slot order, to its tile's mean. Operands that arrive tile-ordered are only pooled.
     {
-        const bool from_tiles = tiled || qkv_is_bf16;
-        const void* const src[3] = {from_tiles ? (const void*)qt : q, from_tiles ? (const void*)kt : k,
-                                    from_tiles ? (const void*)vt : v};
         float* const means[3] = {qc, kc, vc};
-        // tile-ordered input: identity slot map (null), rows per bh = padded
-        e = fv_internal_launch_tile_mean3(src, from_tiles ? 1 : 0, from_tiles ? nullptr : slot_src, block_sizes, means, bh,
-                                          from_tiles ? padded : seq, (int)dim, (int)num_tiles, st);
-        if (e != hipSuccess) return fv_fail_hip(e, "vsa_tile_mean");
+        const void* const src[3] = {q, k, v};
+        if (!tiled) {
+            uint16_t* const tiles[3] = {(uint16_t*)(ws + w.qt), (uint16_t*)(ws + w.kt), (uint16_t*)(ws + w.vt)};
+            e = fv_internal_launch_tile_scan3(src, qkv_is_bf16, slot_src, block_sizes, tiles, means, bh, seq, padded,
+                                              (int)num_tiles, st);
+            qt = tiles[0], kt = tiles[1], vt = tiles[2];
+        } else {
+            e = fv_internal_launch_tile_scan3(src, 1, nullptr, block_sizes, nullptr, means, bh, padded, padded,
+                                              (int)num_tiles, st);
+        }
+        if (e != hipSuccess) return fv_fail_hip(e, "vsa_tile_scan");
     }
     // 2. coarse attention over tiles; raw scores kept for the selection (rt/vsa.rs:385-394)
     if ((rc = fv_vsa_coarse(qc, kc, vc, scores, coarse, bh, num_tiles, dim, scale, stream))) return rc;

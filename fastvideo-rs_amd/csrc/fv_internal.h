@@ -131,12 +131,10 @@ extern "C" hipError_t fv_internal_launch_coarse(const float* qc, const float* kc
                                                 int dim, float scale, hipStream_t st);
 extern "C" hipError_t fv_internal_launch_topk(const float* scores, unsigned* out, int rows, int n, int k,
                                               hipStream_t st);
-extern "C" hipError_t fv_internal_launch_tile_qkv3(const void* const x[3], int x_is_bf16, const int* slot_src,
-                                                   uint16_t* const xt[3], size_t bh, size_t seq, size_t padded, int dim,
-                                                   hipStream_t st);
-extern "C" hipError_t fv_internal_launch_tile_mean3(const void* const x[3], int x_is_bf16, const int* slot_src,
-                                                    const int* block_sizes, float* const out[3], size_t bh, size_t seq,
-                                                    int dim, int num_tiles, hipStream_t st);
+extern "C" hipError_t fv_internal_launch_tile_scan3(const void* const x[3], int x_is_bf16, const int* slot_src,
+                                                    const int* block_sizes, uint16_t* const tiles[3],
+                                                    float* const means[3], size_t bh, size_t seq, size_t padded,
+                                                    int num_tiles, hipStream_t st);
 extern "C" hipError_t fv_internal_launch_tile_qkv(const void* x, int x_is_bf16, const int* slot_src,
                                                   uint16_t* xt, size_t bh, size_t seq, size_t padded,
                                                   int dim, hipStream_t st);

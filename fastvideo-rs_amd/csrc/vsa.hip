@@ -77,17 +77,90 @@ __global__ __launch_bounds__(256) void vsa_tile_mean_kernel(
     int num_tiles, int round16) {
     tile_mean_body<IN_BF16>(x, slot_src, block_sizes, out, seq, dim, num_tiles, round16);
 }
-// q, k and v of the whole op in one launch (blockIdx.z picks the tensor)
-struct Three {
+// ---- tile pass and tile means in one scan (the whole op; rt/vsa.rs:378-384 and 406-414) ----------------
+// dim == 128. 16 lanes per tile, a lane owns 8 consecutive d of every slot: it reads the slot's 16 (bf16) or 32
+// (f32) bytes, writes them as bf16 (RNE) to the tile-ordered copy if there is one (zeros for padding slots), and adds
+// them in f32, in slot order over the tile's real tokens, to its share of the mean: the same values in the same
+// order as vsa_tile_mean_kernel, so the means (and the selection that follows from them) are bit-identical.
+// slot_src == null: x is already tile-ordered. Eight slots in flight per lane. (Measured and not kept: the tile's 64
+// slot indices fetched once and handed round the 16-lane row, the next batch's rows requested before a batch is
+// stored and added: 124 registers and 10 % slower.)
+struct ThreeScan {
     const void* in[3];
-    void* out[3];
+    uint16_t* tiles[3];   // null: no copy wanted
+    float* means[3];
 };
 template <bool IN_BF16>
-__global__ __launch_bounds__(256) void vsa_tile_mean3_kernel(Three t, const int* __restrict__ slot_src,
-                                                             const int* __restrict__ block_sizes, long seq, int dim,
-                                                             int num_tiles, int round16) {
-    tile_mean_body<IN_BF16>(t.in[blockIdx.z], slot_src, block_sizes, (float*)t.out[blockIdx.z], seq, dim, num_tiles,
-                            round16);
+__global__ __launch_bounds__(256) void vsa_tile_scan3_kernel(ThreeScan t, const int* __restrict__ slot_src,
+                                                             const int* __restrict__ block_sizes, long seq, long padded,
+                                                             int num_tiles) {
+    constexpr int kDim = 128;
+    const int grp = threadIdx.x >> 4, c = threadIdx.x & 15;
+    const int tile = blockIdx.x * 16 + grp;
+    if (tile >= num_tiles) return;
+    const long bh = blockIdx.y;
+    const void* __restrict__ x = t.in[blockIdx.z];
+    uint16_t* __restrict__ xt = t.tiles[blockIdx.z];
+    const int n = block_sizes[tile];
+    const long row0 = (long)tile * kTileElems;
+    const int* src = slot_src ? slot_src + row0 : nullptr;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] = 0.f;
+    for (int j = 0; j < kTileElems; j += 8) {
+        float v[8][8];
+        u32x4 packed[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const long tok = src ? (long)src[j + u] : row0 + j + u;
+            const bool real = tok >= 0;
+            if constexpr (IN_BF16) {
+                u32x4 raw = {0u, 0u, 0u, 0u};
+                if (real) raw = *reinterpret_cast<const u32x4*>((const uint16_t*)x + (bh * seq + tok) * kDim + c * 8);
+                packed[u] = raw;
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    v[u][2 * w] = __builtin_bit_cast(float, raw[w] << 16);
+                    v[u][2 * w + 1] = __builtin_bit_cast(float, raw[w] & 0xffff0000u);
+                }
+            } else {
+                f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = a;
+                if (real) {
+                    const float* px = (const float*)x + (bh * seq + tok) * kDim + c * 8;
+                    a = *reinterpret_cast<const f32x4*>(px);
+                    b = *reinterpret_cast<const f32x4*>(px + 4);
+                }
+#pragma unroll
+                for (int w = 0; w < 4; w++) v[u][w] = a[w], v[u][4 + w] = b[w];
+                if (xt) {
+#pragma unroll
+                    for (int w = 0; w < 4; w++)
+                        packed[u][w] = bf16_rne_bits(v[u][2 * w]) | ((unsigned)bf16_rne_bits(v[u][2 * w + 1]) << 16);
+                }
+            }
+        }
+        if (xt) {
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                *reinterpret_cast<u32x4*>(xt + (bh * padded + row0 + j + u) * kDim + c * 8) = packed[u];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            if (j + u < n) {   // uniform over the tile's 16 lanes
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e] = __fadd_rn(acc[e], v[u][e]);
+            }
+        }
+    }
+    float* ob = t.means[blockIdx.z] + (bh * num_tiles + tile) * (long)kDim + c * 8;
+    f32x4 r0, r1;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        r0[e] = n > 0 ? __fdiv_rn(acc[e], (float)n) : 0.0f;
+        r1[e] = n > 0 ? __fdiv_rn(acc[4 + e], (float)n) : 0.0f;
+    }
+    *reinterpret_cast<f32x4*>(ob) = r0;
+    *reinterpret_cast<f32x4*>(ob + 4) = r1;
 }
 
 // ---- coarse scores (rt/vsa.rs:385-388; arithmetic of the host oracle, rt/vsa.rs:185-189) ----
@@ -318,11 +391,6 @@ __global__ __launch_bounds__(256) void vsa_tile_qkv_kernel(const void* __restric
                                                            long padded, int dim) {
     tile_qkv_body<IN_BF16>(x, slot_src, xt, seq, padded, dim);
 }
-template <bool IN_BF16>
-__global__ __launch_bounds__(256) void vsa_tile_qkv3_kernel(Three t, const int* __restrict__ slot_src, long seq,
-                                                            long padded, int dim) {
-    tile_qkv_body<IN_BF16>(t.in[blockIdx.z], slot_src, (uint16_t*)t.out[blockIdx.z], seq, padded, dim);
-}
 
 // ---- fine stage (kernels/core.cu:1029-1179) ---------------------------------------------
 // One workgroup (2 waves x 32 queries) per (query tile, batch*head): online
@@ -542,29 +610,18 @@ extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16,
     return hipGetLastError();
 }
 
-// q, k and v in one launch each for the tile pass and the tile means (the whole op's order: the pass first,
-// the means from its bf16 output when mean_from_tiles, else from the operands where they lie).
-extern "C" hipError_t fv_internal_launch_tile_qkv3(const void* const x[3], int x_is_bf16, const int* slot_src,
-                                                   uint16_t* const xt[3], size_t bh, size_t seq, size_t padded, int dim,
-                                                   hipStream_t st) {
-    Three t;
-    for (int i = 0; i < 3; i++) t.in[i] = x[i], t.out[i] = xt[i];
-    const size_t per = padded * (size_t)(dim / 8);
-    const dim3 grid((unsigned)((per + 255) / 256), (unsigned)bh, 3), block(256);
-    if (x_is_bf16) hipLaunchKernelGGL(vsa_tile_qkv3_kernel<true>, grid, block, 0, st, t, slot_src, (long)seq, (long)padded, dim);
-    else hipLaunchKernelGGL(vsa_tile_qkv3_kernel<false>, grid, block, 0, st, t, slot_src, (long)seq, (long)padded, dim);
-    return hipGetLastError();
-}
-extern "C" hipError_t fv_internal_launch_tile_mean3(const void* const x[3], int x_is_bf16, const int* slot_src,
-                                                    const int* block_sizes, float* const out[3], size_t bh, size_t seq,
-                                                    int dim, int num_tiles, hipStream_t st) {
-    Three t;
-    for (int i = 0; i < 3; i++) t.in[i] = x[i], t.out[i] = out[i];
-    const dim3 grid((num_tiles + 7) / 8, (unsigned)bh, 3), block(256);
+// Tile pass (tiles != null) and tile means of q, k and v in one launch; dim == 128.
+extern "C" hipError_t fv_internal_launch_tile_scan3(const void* const x[3], int x_is_bf16, const int* slot_src,
+                                                    const int* block_sizes, uint16_t* const tiles[3],
+                                                    float* const means[3], size_t bh, size_t seq, size_t padded,
+                                                    int num_tiles, hipStream_t st) {
+    ThreeScan t;
+    for (int i = 0; i < 3; i++) t.in[i] = x[i], t.tiles[i] = tiles ? tiles[i] : nullptr, t.means[i] = means[i];
+    const dim3 grid((num_tiles + 15) / 16, (unsigned)bh, 3), block(256);
     if (x_is_bf16)
-        hipLaunchKernelGGL(vsa_tile_mean3_kernel<true>, grid, block, 0, st, t, slot_src, block_sizes, (long)seq, dim, num_tiles, 0);
+        hipLaunchKernelGGL(vsa_tile_scan3_kernel<true>, grid, block, 0, st, t, slot_src, block_sizes, (long)seq, (long)padded, num_tiles);
     else
-        hipLaunchKernelGGL(vsa_tile_mean3_kernel<false>, grid, block, 0, st, t, slot_src, block_sizes, (long)seq, dim, num_tiles, 0);
+        hipLaunchKernelGGL(vsa_tile_scan3_kernel<false>, grid, block, 0, st, t, slot_src, block_sizes, (long)seq, (long)padded, num_tiles);
     return hipGetLastError();
 }
 
