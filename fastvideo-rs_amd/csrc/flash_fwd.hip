@@ -87,7 +87,7 @@ __device__ unsigned long long g_exact_pass_reruns;
 // this form only for results that are rounded to bf16 anyway.
 template <bool MASKED, int D, bool LOG2DOM, bool FIXED, class Params>
 FV_DEV bool flash_item(const Params& p, const int wave, const int lane, const int block) {
-    // (masked launches: only where every query sees a key among the walk's first 128, see launch_flash)
+    // (masked launches: only where every query sees key 0, see launch_flash)
     using G = TileGeo<D>;
     constexpr int kD = D;
     constexpr int kTileBytes = G::kTile;
@@ -635,13 +635,13 @@ hipError_t launch_flash_fixed(const fv::FlashParams* p, hipStream_t stream) {
 }
 // Launches whose result is rounded to bf16 make their first pass with the fixed offset: on a row that one late
 // key dominates, that key's P is then a rounded bf16 number instead of exactly 1 (up to 2^-8 relative on the row),
-// which a bf16 result absorbs; f32 results keep the running max. Masked launches take it where every query sees a
-// key among the first 128 of its tile's walk, so that its offset is a score of its own: block-causal without a
-// window (key 0 is visible to every query). Under a window, or the VDN mask, a query's first visible key may lie
-// anywhere in the walk: those keep the running max.
+// which a bf16 result absorbs; f32 results keep the running max. Masked launches take it where every query sees
+// key 0, the first key of every tile's walk, so that its offset is a score of its own: block-causal without a
+// window or with sink blocks, and the VDN mask (rows before the video and frame 0 are visible to every query).
+// Under a window without a sink a query's first visible key may lie anywhere in the walk: running max.
 template <bool MASKED, int D>
 hipError_t launch_flash(const fv::FlashParams* p, hipStream_t stream) {
-    const bool offset_is_a_score = !MASKED || (p->mask_mode == 1 && p->win == 0);
+    const bool offset_is_a_score = !MASKED || p->mask_mode == 2 || (p->mask_mode == 1 && (p->win == 0 || p->sink > 0));
     if (p->out_is_bf16 && offset_is_a_score && !running_max_forced()) return launch_flash_fixed<MASKED, D, true>(p, stream);
     return launch_flash_fixed<MASKED, D, false>(p, stream);
 }

@@ -8,7 +8,7 @@ anchor ranges, and the degenerate clips (1-2 frames, radius past the clip) that 
 import numpy as np
 import pytest
 
-from util import announce, assert_parity, qkv, to_dev_bf16
+from util import announce, assert_bf16_result_matches_f32_result, assert_parity, qkv, to_dev_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -50,7 +50,45 @@ def test_vdn_window_matches_masked_oracle(fv, oracle, bh, s, vs, t, frames, chun
     assert_parity(got, want, f"vdn_{s}_{vs}_{t}x{frames}_c{chunk}_r{radius}")
     got16 = fv.sdpa_vdn_window_bf16(qd, kd, vd, vs, t, frames, chunk, radius, out_bf16=True)
     torch.cuda.synchronize()
-    assert np.array_equal(got16.float().cpu().numpy(), oracle.quantize_bf16(got))
+    # (the bf16 launch keeps its softmax offset fixed after the first 128 keys, the f32 one follows the running max)
+    assert_bf16_result_matches_f32_result(got16.float().cpu().numpy(), got, f"vdn_{s}_{vs}_{t}x{frames}", exact_share=0.999)
+
+
+def test_fixed_offset_pass_under_the_window_and_its_rerun(fv, oracle):
+    """Every query sees key 0 under this mask (rows before the video and frame 0 are visible to all), so launches
+    that write bf16 fix each query's softmax offset at the largest score of its walk's first 128 keys and redo the
+    pass with the running max where a row outgrew it. Head 0's scores climb by hundreds of base-2 units along the
+    keys: its workgroups take the second pass (counted), every row matches the masked f32 host math, and the other
+    head is the bits of a launch on its own."""
+    import torch
+
+    bh, s, d = 2, 1300, 128
+    vs, t, frames, chunk, radius = 20, 40, 32, 5, 1
+    announce("vdn window fixed-offset pass and its rerun")
+    rng = np.random.Generator(np.random.PCG64(909))
+    q = rng.standard_normal((bh, s, d)).astype(np.float32)
+    k = rng.standard_normal((bh, s, d)).astype(np.float32)
+    v = oracle.quantize_bf16(rng.standard_normal((bh, s, d)).astype(np.float32))
+    q[0] = np.abs(q[0]) + 2.0
+    k[0, :128] = -0.5
+    k[0, 128:] = np.linspace(1.0, 30.0, s - 128, dtype=np.float32)[:, None]
+    q, k = oracle.quantize_bf16(q), oracle.quantize_bf16(k)
+    tq, tk, tv = (to_dev_bf16(x) for x in (q, k, v))
+    lib = fv.lib()
+    n0 = lib.fv_sdpa_exact_pass_reruns()
+    got = fv.sdpa_vdn_window_bf16(tq, tk, tv, vs, t, frames, chunk, radius, out_bf16=True)
+    torch.cuda.synchronize()
+    n1 = lib.fv_sdpa_exact_pass_reruns()
+    assert n1 - n0 == (s + 255) // 256, (n0, n1)       # every query tile of head 0 sees keys past its first 128
+    mask = oracle.vdn_window_dense_mask(vs, t, frames, chunk, radius, s, s)
+    want = oracle.sdpa_composed(q, k, v, mask=mask)
+    assert_parity(got.float().cpu().numpy(), want, "vdn_rerun", max_abs=2e-2)
+    rest = fv.sdpa_vdn_window_bf16(tq[1:].contiguous(), tk[1:].contiguous(), tv[1:].contiguous(), vs, t, frames, chunk,
+                                   radius, out_bf16=True)
+    got32 = fv.sdpa_vdn_window_bf16(tq, tk, tv, vs, t, frames, chunk, radius)
+    torch.cuda.synchronize()
+    assert lib.fv_sdpa_exact_pass_reruns() == n1 and torch.equal(rest, got[1:])   # f32 results keep the running max
+    assert_parity(got32.cpu().numpy(), want, "vdn_running_max")
 
 
 def test_masked_rows_really_differ_from_dense(fv, oracle):
