@@ -524,7 +524,7 @@ FV_DEV bool flash_item(const Params& p, const int wave, const int lane, const in
 
 // The softmax offset rides in the C operand of the K Q^T MFMAs (softmax_tile_pair_off): a score costs one multiply,
 // one exponential and one add. LOG2DOM: the call's scale * log2(e) is exactly 1 (scores are base-2 logarithms as
-// they leave the MFMAs) and the multiply is gone too. FIXED (dense launches that write bf16): the first pass keeps
+// they leave the MFMAs) and the multiply is gone too. FIXED (launches that write bf16 and whose queries all see key 0): the first pass keeps
 // the offset of the first 128 keys (flash_item); the others keep the running max throughout.
 template <bool MASKED, int D, bool LOG2DOM, bool FIXED>
 __global__ __launch_bounds__(512, 2) void flash_fwd_pp2(const FlashParams p) {

@@ -77,7 +77,7 @@ def sample_rows(seed, sq, n, extra=()):
 
 
 def assert_bf16_result_matches_f32_result(got16, got32, tag, exact_share=0.0):
-    """A launch that writes bf16 against the same launch writing f32. Dense launches that write bf16 keep their softmax
+    """A launch that writes bf16 against the same launch writing f32. Launches that write bf16 (and whose queries all see key 0) keep their softmax
     offset fixed after the first 128 keys where the f32 ones follow the running max: the same arithmetic, hence the
     RNE rounding of the f32 result bit for bit, for every wave in which no row's maximum grows by 2^6 after its first
     128 keys; two roundings of P apart otherwise (each about 1.6e-3 of the result's rms in l2, several times that at
