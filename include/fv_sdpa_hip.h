@@ -60,8 +60,9 @@ int fv_sdpa_is_log2_domain_scale(float scale);
 /* Launches of that form of the dense / masked kernel since the library was loaded (all its entries together). */
 uint64_t fv_sdpa_log2_domain_launches(void);
 
-/* No counterpart in the reference (a diagnostic). Dense launches make their pass over the keys with every query's
- * softmax offset fixed at the largest score of its first 128 keys (no running max in the loop), check the row sums
+/* No counterpart in the reference (a diagnostic). Launches that write bf16 and in which every query sees key 0
+ * (dense; block-causal without a window or with sink blocks; the VDN window) make their pass over the keys with every
+ * query's softmax offset fixed at the largest score of its first 128 keys (no running max in the loop), check the row sums
  * and accumulators before anything is stored, and make the pass again with the running max in any workgroup where
  * a row's scores outgrew that offset by more than about 2^60: results are exact either way, the second pass only
  * costs time. This is the number of workgroups that took it on the current device since the library was loaded.
@@ -133,7 +134,9 @@ int fv_sdpa_dense_bf16_splitkv_static(const uint16_t* q, const uint16_t* k, cons
  * Key tiles no query of a workgroup can see are never loaded. A query that sees no key at all (more queries than
  * keys under a window that has moved past the last key) gets a row of zeros, what the reference's fused kernel
  * stores for a row without a visible key (kernels/attn2.cu:150); its composed route with the additive -1e9 mask
- * (rt/attn.rs:455-467) would give such a row the mean of V. No reference fixture covers the case: parity unpinned. */
+ * (rt/attn.rs:455-467) would give such a row the mean of V. No reference fixture covers the case: parity unpinned.
+ * Rounding of bf16 results as for fv_sdpa_dense_bf16 when every query sees key 0 (window == 0 or sink > 0); under a
+ * window without a sink every row follows its running maximum. */
 int fv_sdpa_block_causal_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                               int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d,
                               float scale, size_t block_tokens, size_t window, size_t sink,
@@ -144,7 +147,8 @@ int fv_sdpa_block_causal_bf16(const uint16_t* q, const uint16_t* k, const uint16
  * fv_vdn_window_allows): a key-tile walk over at most three ranges per query tile (rows before the
  * video + frame 0, the window frames of the tile, the last frame + rows after the video), per-score
  * masking on boundary tiles only. Self-attention (sq == sk), frames > 0, frame_tokens > 0, the video
- * rows inside the sequence; otherwise declines. */
+ * rows inside the sequence; otherwise declines. Rounding of bf16 results as for fv_sdpa_dense_bf16 (every query
+ * sees key 0 under this mask). */
 int fv_sdpa_vdn_window_bf16(const uint16_t* q, const uint16_t* k, const uint16_t* v, void* out,
                             int out_is_bf16, size_t bh, size_t sq, size_t sk, size_t d, float scale,
                             size_t video_start, size_t frame_tokens, size_t frames, size_t chunk,
