@@ -213,6 +213,65 @@ __global__ __launch_bounds__(64) void vsa_tile_scan3_staged_kernel(ThreeScan t, 
     *reinterpret_cast<float2*>(ob) = r;
 }
 
+// ... and for f32 operands: the tile in two halves of 32 slots (16 KB of f32 each), two consecutive slots per load
+// instruction; the copy is rounded to bf16 (RNE), the sums take the unrounded values, lane c owning d = c and c + 64.
+__global__ __launch_bounds__(64) void vsa_tile_scan3_staged_f32_kernel(ThreeScan t, const int* __restrict__ slot_src,
+                                                                       const int* __restrict__ block_sizes, long seq,
+                                                                       long padded, int num_tiles) {
+    __shared__ __attribute__((aligned(16))) unsigned stage[32 * 128];   // 32 rows x 128 words
+    const int lane = threadIdx.x;
+    const int tile = blockIdx.x;
+    const long bh = blockIdx.y;
+    const float* __restrict__ x = (const float*)t.in[blockIdx.z];
+    uint16_t* __restrict__ xt = t.tiles[blockIdx.z];
+    const long row0 = (long)tile * kTileElems;
+    const int n = block_sizes[tile];
+    const int my_tok = slot_src ? slot_src[row0 + lane] : (int)(row0 + lane);   // lane = slot
+    const int c = lane & 31;
+    float a0 = 0.f, a1 = 0.f;
+    u32x4 v[2][16];
+    auto load_half = [&](int half, u32x4 (&r)[16]) {
+#pragma unroll
+        for (int it = 0; it < 16; it++) {
+            const int slot = 32 * half + it * 2 + (lane >> 5);
+            const int tok = __shfl(my_tok, slot);
+            r[it] = u32x4{0u, 0u, 0u, 0u};
+            if (tok >= 0) r[it] = *reinterpret_cast<const u32x4*>(x + (bh * seq + tok) * 128 + c * 4);
+        }
+    };
+    load_half(0, v[0]);
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        if (half == 0) load_half(1, v[1]);   // in flight while the first half is stored and added
+#pragma unroll
+        for (int it = 0; it < 16; it++) {
+            const int sl = it * 2 + (lane >> 5);
+            const u32x4 w = v[half][it];
+            // (the vector cast as a whole: __builtin_bit_cast(float, w[i]) read element 0 for every i with hipcc 7.2)
+            const f32x4 f = __builtin_bit_cast(f32x4, w);
+            u32x2 packed;
+            packed[0] = bf16_rne_bits(f[0]) | ((unsigned)bf16_rne_bits(f[1]) << 16);
+            packed[1] = bf16_rne_bits(f[2]) | ((unsigned)bf16_rne_bits(f[3]) << 16);
+            *reinterpret_cast<u32x2*>(xt + (bh * padded + row0 + 32 * half + sl) * 128 + c * 4) = packed;
+            *reinterpret_cast<u32x4*>(&stage[sl * 128 + c * 4]) = w;
+        }
+        __syncthreads();   // one wave: orders its LDS writes before the reads below
+#pragma unroll 8
+        for (int j = 0; j < 32; j++) {
+            const float w0 = __builtin_bit_cast(float, stage[j * 128 + lane]);
+            const float w1 = __builtin_bit_cast(float, stage[j * 128 + 64 + lane]);
+            if (32 * half + j < n) {
+                a0 = __fadd_rn(a0, w0);
+                a1 = __fadd_rn(a1, w1);
+            }
+        }
+        __syncthreads();   // ... and the reads before the next half's writes
+    }
+    float* ob = t.means[blockIdx.z] + (bh * num_tiles + tile) * 128L;
+    ob[lane] = n > 0 ? __fdiv_rn(a0, (float)n) : 0.0f;
+    ob[64 + lane] = n > 0 ? __fdiv_rn(a1, (float)n) : 0.0f;
+}
+
 // ---- coarse scores (rt/vsa.rs:385-388; arithmetic of the host oracle, rt/vsa.rs:185-189) ----
 // scores[bh, qt, kt] = f32( (f64 dot of the tile means, d ascending from -0.0) * f64(scale) ).
 // The product of two f32 values is exact in f64, so one v_fma_f64 per term is the oracle's
@@ -668,9 +727,13 @@ extern "C" hipError_t fv_internal_launch_tile_scan3(const void* const x[3], int 
     ThreeScan t;
     for (int i = 0; i < 3; i++) t.in[i] = x[i], t.tiles[i] = tiles ? tiles[i] : nullptr, t.means[i] = means[i];
     const dim3 grid((num_tiles + 15) / 16, (unsigned)bh, 3), block(256);
-    if (x_is_bf16 && tiles) {
-        hipLaunchKernelGGL(vsa_tile_scan3_staged_kernel, dim3(num_tiles, (unsigned)bh, 3), dim3(64), 0, st, t, slot_src,
-                           block_sizes, (long)seq, (long)padded, num_tiles);
+    if (tiles) {
+        if (x_is_bf16)
+            hipLaunchKernelGGL(vsa_tile_scan3_staged_kernel, dim3(num_tiles, (unsigned)bh, 3), dim3(64), 0, st, t, slot_src,
+                               block_sizes, (long)seq, (long)padded, num_tiles);
+        else
+            hipLaunchKernelGGL(vsa_tile_scan3_staged_f32_kernel, dim3(num_tiles, (unsigned)bh, 3), dim3(64), 0, st, t,
+                               slot_src, block_sizes, (long)seq, (long)padded, num_tiles);
         return hipGetLastError();
     }
     if (x_is_bf16)
