@@ -80,7 +80,7 @@ __device__ unsigned long long g_exact_pass_reruns;
 // stays there: no row max and no rescale decision in the loop (32 three-operand VALU instructions a phase less:
 // 2 % of the time of the long launches, 9 % at head dim 64). Exact for any input as long as nothing overflows (P
 // and l share the offset), so the pass is checked before anything is stored: if some row's scores grew by more
-// than about 2^60 past that first maximum (a row sum outside the comfortable f32 range, or an accumulator not
+// than about 2^90 past that first maximum (a row sum of 2^100 or more, whose reciprocal nears the subnormals, or an accumulator not
 // finite), the workgroup makes the pass again from the top with the running max. One difference in rounding
 // remains: the largest P of a row is exactly 1 under the running max and a rounded bf16 number under the fixed
 // offset, so a row that ONE late key dominates can be off by up to 2^-8 relative; the launcher therefore takes
@@ -428,14 +428,14 @@ FV_DEV bool flash_item(const Params& p, const int wave, const int lane, const in
     pv_tile<D>(vbuf(2 * np - 1), rb.v, pb1, o);
 
     if constexpr (FIXED) {
-        // Did the fixed offset hold? Every row sum comfortably inside the f32 range and every accumulator finite
+        // Did the fixed offset hold? Every row sum below 2^100 (its reciprocal a normal number with room to spare) and every accumulator finite
         // (x * 0 is NaN for an infinite or NaN x). One vote per wave through 8 words of LDS behind the rings.
         float chk = 0.f;
 #pragma unroll
         for (int db = 0; db < kNO; db++)
 #pragma unroll
             for (int i = 0; i < 16; i++) chk = __builtin_fmaf(o[db][i], 0.f, chk);
-        const bool lane_ok = (pair_sum(st.l_acc) < 0x1p+64f) && (chk == 0.f);
+        const bool lane_ok = (pair_sum(st.l_acc) < 0x1p+100f) && (chk == 0.f);
         auto* votes = (__attribute__((address_space(3))) unsigned*)(smem + 2 * kRing2 * kTileBytes);
         if (lane == 0) votes[wave] = __builtin_amdgcn_ballot_w64(!lane_ok) != 0 ? 1u : 0u;
         __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the vote is written before the barrier

@@ -64,7 +64,7 @@ uint64_t fv_sdpa_log2_domain_launches(void);
  * (dense; block-causal without a window or with sink blocks; the VDN window) make their pass over the keys with every
  * query's softmax offset fixed at the largest score of its first 128 keys (no running max in the loop), check the row sums
  * and accumulators before anything is stored, and make the pass again with the running max in any workgroup where
- * a row's scores outgrew that offset by more than about 2^60: results are exact either way, the second pass only
+ * a row's scores outgrew that offset by more than about 2^90: results are exact either way, the second pass only
  * costs time. This is the number of workgroups that took it on the current device since the library was loaded.
  * Blocks until the device's work so far is done (a device-to-host copy of the counter); 0 without a device. */
 uint64_t fv_sdpa_exact_pass_reruns(void);

@@ -216,7 +216,7 @@ def test_full_size_prefix_and_block_properties(fv, bt, win, sink):
 def test_block_causal_pass_with_the_fixed_offset_and_its_rerun(fv, oracle, d):
     """Block-causal launches that write bf16 and in which every query sees key 0 (no window, or sink blocks) make their
     pass with every query's softmax offset fixed at the largest score among the first 128 keys of its tile's walk and
-    redo it with the running max where a row outgrew that by more than about 2^60. One head's later keys score hundreds of base-2
+    redo it with the running max where a row outgrew that by more than about 2^90. One head's later keys score hundreds of base-2
     units above its first ones: its workgroups take the second pass (counted), every row matches the f64 host math
     under the mask, the other heads' rows are the bits of a launch without that head; a launch under a window
     with a sink block does the same, and one under a window without a sink (whose queries may see none of the walk's

@@ -323,7 +323,7 @@ def test_extreme_score_ranges(fv, oracle, d):
 @pytest.mark.parametrize("out_bf16", [False, True])
 def test_scores_that_outgrow_the_first_maximum_redo_the_pass(fv, oracle, d, out_bf16):
     """Dense launches that write bf16 fix every query's softmax offset at the largest score of its first 128 keys and
-    verify afterwards; a workgroup whose scores grew by more than about 2^60 past it makes its pass again with the
+    verify afterwards; a workgroup whose scores grew by more than about 2^90 past it makes its pass again with the
     running max (launches that write f32 keep the running max throughout). Here the keys past the first 128 score
     hundreds of base-2 units above the first ones for one head (the fixed offset overflows: P = inf), mildly above
     for another (no rerun needed), and as usual for the third: every row must match the f64 host math, the rerun
