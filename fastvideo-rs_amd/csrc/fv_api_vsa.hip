@@ -331,6 +331,7 @@ static int vsa_attention_common(const void* q, const void* k, const void* v, int
     hipStream_t st = (hipStream_t)stream;
     hipError_t e;
     int rc;
+    bool fold = false;
     // 1 + 4. tile means (rt/vsa.rs:378-384) and the tile-ordered bf16 copies for the fine stage (rt/vsa.rs:406-414)
     //    of q, k and v in ONE scan: every token row is read once, written to its slot as bf16 and added, unrounded
     //    and in slot order, to its tile's mean. Operands that arrive tile-ordered are only pooled.
@@ -339,11 +340,16 @@ static int vsa_attention_common(const void* q, const void* k, const void* v, int
         const void* const src[3] = {q, k, v};
         if (!tiled) {
             uint16_t* const tiles[3] = {(uint16_t*)(ws + w.qt), (uint16_t*)(ws + w.kt), (uint16_t*)(ws + w.vt)};
-            e = fv_internal_launch_tile_scan3(src, qkv_is_bf16, slot_src, block_sizes, tiles, means, bh, seq, padded,
-                                              (int)num_tiles, st);
+            // f32 queries get their one rounding here: with the fold switch on (fv_rt_fold_scale), of
+            // q * (scale * log2 e), and the fine kernel then runs its form without the per-score multiply
+            const float c = scale * 1.4426950408889634f;
+            const float copy_mul[3] = {c, 1.0f, 1.0f};
+            fold = !qkv_is_bf16 && fv_rt_fold_scale() && c != 1.0f && c < 3.0e38f;
+            e = fv_internal_launch_tile_scan3(src, qkv_is_bf16, slot_src, block_sizes, tiles, means,
+                                              fold ? copy_mul : nullptr, bh, seq, padded, (int)num_tiles, st);
             qt = tiles[0], kt = tiles[1], vt = tiles[2];
         } else {
-            e = fv_internal_launch_tile_scan3(src, 1, nullptr, block_sizes, nullptr, means, bh, padded, padded,
+            e = fv_internal_launch_tile_scan3(src, 1, nullptr, block_sizes, nullptr, means, nullptr, bh, padded, padded,
                                               (int)num_tiles, st);
         }
         if (e != hipSuccess) return fv_fail_hip(e, "vsa_tile_scan");
@@ -363,7 +369,7 @@ static int vsa_attention_common(const void* q, const void* k, const void* v, int
     p.out = nullptr;
     p.num_tiles = (int)num_tiles;
     p.topk = (int)topk;
-    p.sl2 = scale * 1.4426950408889634f;
+    p.sl2 = fold ? 1.0f : scale * 1.4426950408889634f;
     p.q_base = 0;
     p.q_tiles = (int)num_tiles;
     p.total = (int)(bh * num_tiles);

@@ -133,8 +133,8 @@ extern "C" hipError_t fv_internal_launch_topk(const float* scores, unsigned* out
                                               hipStream_t st);
 extern "C" hipError_t fv_internal_launch_tile_scan3(const void* const x[3], int x_is_bf16, const int* slot_src,
                                                     const int* block_sizes, uint16_t* const tiles[3],
-                                                    float* const means[3], size_t bh, size_t seq, size_t padded,
-                                                    int num_tiles, hipStream_t st);
+                                                    float* const means[3], const float* copy_mul, size_t bh, size_t seq,
+                                                    size_t padded, int num_tiles, hipStream_t st);
 extern "C" hipError_t fv_internal_launch_tile_qkv(const void* x, int x_is_bf16, const int* slot_src,
                                                   uint16_t* xt, size_t bh, size_t seq, size_t padded,
                                                   int dim, hipStream_t st);

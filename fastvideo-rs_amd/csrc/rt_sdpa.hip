@@ -248,8 +248,9 @@ Result<std::optional<Tensor>> fused(const Tensor& q, const Tensor& k, const Tens
                                     const VdnWindow* window = nullptr) {
     const auto s = bhsd(q, k, v);
     if (!s || !fv_sdpa_supported(s->b, s->h, s->sq, s->sk, s->d)) return std::optional<Tensor>{};
-    // f32 queries are rounded to bf16 here, once: with the fold switch on, of q * (scale * log2(e)), and the
-    // kernel then runs at scale = ln 2, its form without the per-score multiply-add
+    // f32 queries are rounded to bf16 here, once: with the fold switch on (off by default: the result then differs
+    // from the reference's round-then-scale order by one rounding of q), of q * (scale * log2(e)), and the
+    // kernel then runs at scale = ln 2, its form without the per-score multiply
     float sc = default_scale(scale, s->d);
     float q_mul = 1.0f;
     if (q.dtype == DType::F32 && fold_scale()) {
@@ -549,7 +550,7 @@ bool causal_flash_enabled() {
 }
 bool fold_scale() {
     if (g_fold_override) return *g_fold_override;
-    static const bool env = env_flag("FASTVIDEO_SDPA_FOLD_SCALE", true);
+    static const bool env = env_flag("FASTVIDEO_SDPA_FOLD_SCALE", false);
     return env;
 }
 void set_fold_scale_override(std::optional<bool> v) { g_fold_override = v; }

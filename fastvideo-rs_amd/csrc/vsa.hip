@@ -89,6 +89,8 @@ struct ThreeScan {
     const void* in[3];
     uint16_t* tiles[3];   // null: no copy wanted
     float* means[3];
+    float mul[3];         // f32 operands: factor on the values of the copy before their one rounding (1 = none);
+                          // the means pool the operand as it is
 };
 template <bool IN_BF16>
 __global__ __launch_bounds__(256) void vsa_tile_scan3_kernel(ThreeScan t, const int* __restrict__ slot_src,
@@ -133,9 +135,10 @@ __global__ __launch_bounds__(256) void vsa_tile_scan3_kernel(ThreeScan t, const 
 #pragma unroll
                 for (int w = 0; w < 4; w++) v[u][w] = a[w], v[u][4 + w] = b[w];
                 if (xt) {
+                    const float m = t.mul[blockIdx.z];
 #pragma unroll
                     for (int w = 0; w < 4; w++)
-                        packed[u][w] = bf16_rne_bits(v[u][2 * w]) | ((unsigned)bf16_rne_bits(v[u][2 * w + 1]) << 16);
+                        packed[u][w] = bf16_rne_bits(v[u][2 * w] * m) | ((unsigned)bf16_rne_bits(v[u][2 * w + 1] * m) << 16);
                 }
             }
         }
@@ -228,6 +231,7 @@ __global__ __launch_bounds__(64) void vsa_tile_scan3_staged_f32_kernel(ThreeScan
     const int n = block_sizes[tile];
     const int my_tok = slot_src ? slot_src[row0 + lane] : (int)(row0 + lane);   // lane = slot
     const int c = lane & 31;
+    const float mul = t.mul[blockIdx.z];   // x * 1.0f is x
     float a0 = 0.f, a1 = 0.f;
     u32x4 v[2][16];
     auto load_half = [&](int half, u32x4 (&r)[16]) {
@@ -250,8 +254,8 @@ __global__ __launch_bounds__(64) void vsa_tile_scan3_staged_f32_kernel(ThreeScan
             // (the vector cast as a whole: __builtin_bit_cast(float, w[i]) read element 0 for every i with hipcc 7.2)
             const f32x4 f = __builtin_bit_cast(f32x4, w);
             u32x2 packed;
-            packed[0] = bf16_rne_bits(f[0]) | ((unsigned)bf16_rne_bits(f[1]) << 16);
-            packed[1] = bf16_rne_bits(f[2]) | ((unsigned)bf16_rne_bits(f[3]) << 16);
+            packed[0] = bf16_rne_bits(f[0] * mul) | ((unsigned)bf16_rne_bits(f[1] * mul) << 16);
+            packed[1] = bf16_rne_bits(f[2] * mul) | ((unsigned)bf16_rne_bits(f[3] * mul) << 16);
             *reinterpret_cast<u32x2*>(xt + (bh * padded + row0 + 32 * half + sl) * 128 + c * 4) = packed;
             *reinterpret_cast<u32x4*>(&stage[sl * 128 + c * 4]) = w;
         }
@@ -719,13 +723,16 @@ extern "C" hipError_t fv_internal_launch_tile_mean(const void* x, int x_is_bf16,
     return hipGetLastError();
 }
 
-// Tile pass (tiles != null) and tile means of q, k and v in one launch; dim == 128.
+// Tile pass (tiles != null) and tile means of q, k and v in one launch; dim == 128. copy_mul (f32 operands only,
+// null = none): factors on the values of the three copies before their rounding to bf16.
 extern "C" hipError_t fv_internal_launch_tile_scan3(const void* const x[3], int x_is_bf16, const int* slot_src,
                                                     const int* block_sizes, uint16_t* const tiles[3],
-                                                    float* const means[3], size_t bh, size_t seq, size_t padded,
-                                                    int num_tiles, hipStream_t st) {
+                                                    float* const means[3], const float* copy_mul, size_t bh, size_t seq,
+                                                    size_t padded, int num_tiles, hipStream_t st) {
+    if (copy_mul && x_is_bf16) return hipErrorInvalidValue;   // a second rounding of values already rounded
     ThreeScan t;
-    for (int i = 0; i < 3; i++) t.in[i] = x[i], t.tiles[i] = tiles ? tiles[i] : nullptr, t.means[i] = means[i];
+    for (int i = 0; i < 3; i++)
+        t.in[i] = x[i], t.tiles[i] = tiles ? tiles[i] : nullptr, t.means[i] = means[i], t.mul[i] = copy_mul ? copy_mul[i] : 1.0f;
     const dim3 grid((num_tiles + 15) / 16, (unsigned)bh, 3), block(256);
     if (tiles) {
         if (x_is_bf16)

@@ -222,12 +222,15 @@ int fv_rt_free(void* p, void* stream);
 void fv_rt_set_bf16_activations(int v);
 int fv_rt_bf16_activations(void);
 /* No counterpart in the reference. When q arrives as f32, fv_rt_sdpa itself makes the bf16 copy the fused
- * kernels read (rt/sdpa.rs:167-181 `act16_operands`, rt/attn.rs:283-300): with this switch on (the default;
- * FASTVIDEO_SDPA_FOLD_SCALE=0 turns it off, fv_rt_set_fold_scale overrides per thread, v < 0 clears) that one
- * rounding is taken of q * (scale * log2(e)) and the kernel runs at FV_SDPA_SCALE_LOG2_DOMAIN, the form without
- * the per-score multiply-add. Q is still rounded once, from the same f32 values, so the result is as close to
- * the f32 host math as with the switch off (bf16(c q) in place of c bf16(q): different last bits, same error
- * size); bf16 queries are never touched. Off reproduces the reference's order (round, then scale) exactly. */
+ * kernels read (rt/sdpa.rs:167-181 `act16_operands`, rt/attn.rs:283-300): with this switch on
+ * (FASTVIDEO_SDPA_FOLD_SCALE=1; fv_rt_set_fold_scale overrides per thread, v < 0 clears) that one rounding is
+ * taken of q * (scale * log2(e)) and the kernel runs at FV_SDPA_SCALE_LOG2_DOMAIN, the form without the per-score
+ * multiply; fv_vsa_attention does the same with an f32 q in its tile pass. Q is still rounded once, from the same
+ * f32 values, so the result is as close to the f32 host math as with the switch off (bf16(c q) in place of
+ * c bf16(q): different last bits, same error size) -- but it is one rounding of q away from the host math on the
+ * ROUNDED operands, which is what the reference's own check of its kernel compares with at rel_l2 <= 2e-3
+ * (gpucheck/src/kernels.rs:2314-2320): measured 2.6 - 2.8e-3 with the switch on, 1.3 - 1.6e-3 off. Hence OFF by
+ * default: the reference's order (round, then scale) exactly. bf16 queries are never touched. */
 void fv_rt_set_fold_scale(int v);
 int fv_rt_fold_scale(void);
 /* rt/log.rs:17-37: the level FASTVIDEO_LOG selects (read once): 0 quiet ("0", "off", "false", "quiet",

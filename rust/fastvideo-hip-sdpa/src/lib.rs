@@ -447,9 +447,9 @@ fn fused(q: &CudaTensor, k: &CudaTensor, v: &CudaTensor, scale: Option<f32>, out
     if !mma_sdpa_supported(b, h, sq, sk, d) {
         return Ok(None);
     }
-    // the fused kernels read bf16; f32 operands are rounded once (RNE), as the reference does. An f32 q is
-    // rounded as q * (scale * log2(e)) and the kernel then runs at ln 2, its form without the per-score
-    // multiply-add (fv_rt_fold_scale: on unless FASTVIDEO_SDPA_FOLD_SCALE=0).
+    // the fused kernels read bf16; f32 operands are rounded once (RNE), as the reference does. With the fold
+    // switch on (fv_rt_fold_scale: FASTVIDEO_SDPA_FOLD_SCALE=1, off by default) an f32 q is rounded as
+    // q * (scale * log2(e)) and the kernel then runs at ln 2, its form without the per-score multiply.
     let mut scale = scale.unwrap_or(1.0 / (d as f32).sqrt());
     let mut q_mul = 1.0f32;
     // SAFETY: reads a per-thread flag / host arithmetic only.

@@ -143,9 +143,51 @@ def test_dense_plan_reaches_the_fused_kernel(fv, oracle, act16, f32_in):
                   max_abs=2e-2 if act16 else 1e-2)
 
 
+REFERENCE_SHAPES = [  # (b, h, sq, sk, d, std): gpucheck/src/kernels.rs:2287-2298
+    (1, 1, 1, 1, 128, 1.0), (1, 2, 64, 64, 128, 1.0), (1, 2, 70, 70, 64, 1.0), (2, 3, 257, 257, 128, 1.0),
+    (1, 4, 300, 512, 128, 1.0), (2, 2, 1000, 333, 64, 1.0), (1, 3, 130, 1, 128, 1.0), (1, 2, 63, 4097, 128, 1.0),
+    (2, 2, 1024, 1024, 128, 2.0), (1, 2, 2048, 2048, 128, 1.0),
+]
+
+
+@pytest.mark.parametrize("b,h,sq,sk,d,std", REFERENCE_SHAPES)
+def test_f32_operands_meet_the_reference_bars_in_the_default_order(fv, oracle, b, h, sq, sk, d, std):
+    """The reference's own check of its fused kernel (gpucheck/src/kernels.rs:2286-2328), as it would run against this
+    library: f32 tensors of N(0, std) go to the one entry, which rounds them to bf16 itself; the f32 result is
+    compared with the host math on the f32 operands (rel_l2 <= 1e-2) AND on the operands rounded to bf16 the plain
+    way (<= 2e-3), the bf16 result with the former (<= 1e-2). The default (round, then scale) meets all three; with
+    the scale folded into q's rounding the first and third hold as well, the second cannot (a different rounding of
+    q than the one it assumes) and is only reported."""
+    import torch
+
+    announce(f"rt sdpa on f32 operands, reference bars, {b}x{h}x{sq}x{sk}x{d} std={std}")
+    rng = np.random.Generator(np.random.PCG64(2286 + sq + d))
+    q = rng.standard_normal((b * h, sq, d), dtype=np.float32) * np.float32(std)
+    k = rng.standard_normal((b * h, sk, d), dtype=np.float32) * np.float32(std)
+    v = rng.standard_normal((b * h, sk, d), dtype=np.float32)
+    want = oracle.sdpa_f64(q, k, v)
+    want_rounded = oracle.sdpa_f64(*(oracle.quantize_bf16(x) for x in (q, k, v)))
+    tq, tk, tv = (dev(x.reshape(b, h, -1, d)) for x in (q, k, v))
+    host = lambda t: t.float().cpu().numpy().reshape(b * h, sq, d)
+    assert not fv.fold_scale()
+    with fv.with_bf16_act(False):
+        got = host(fv.sdpa(tq, tk, tv, fv.Plan.dense(None)))
+        with fv.with_fold_scale(True):
+            folded = host(fv.sdpa(tq, tk, tv, fv.Plan.dense(None)))
+    with fv.with_bf16_act(True):
+        got16 = host(fv.sdpa(tq, tk, tv, fv.Plan.dense(None)))
+    torch.cuda.synchronize()
+    m_f32, m_rounded, m16 = metrics(got, want), metrics(got, want_rounded), metrics(got16, want)
+    f_f32, f_rounded = metrics(folded, want), metrics(folded, want_rounded)
+    print(f"[reference bars] vs f32 operands {m_f32['rel_l2']:.3e} (folded {f_f32['rel_l2']:.3e}), vs rounded operands "
+          f"{m_rounded['rel_l2']:.3e} (folded {f_rounded['rel_l2']:.3e}), bf16 result {m16['rel_l2']:.3e}", flush=True)
+    assert m_f32["rel_l2"] <= 1e-2 and m_rounded["rel_l2"] <= 2e-3 and m16["rel_l2"] <= 1e-2
+    assert f_f32["rel_l2"] <= 1e-2
+
+
 @pytest.mark.parametrize("kind", ["dense", "dense_scale", "block_causal", "kv_window"])
 def test_f32_queries_take_the_scale_into_their_one_rounding(fv, oracle, kind):
-    """An f32 q is rounded to bf16 by the library itself (rt/sdpa.rs:167-181): with the fold switch on (default) that
+    """An f32 q is rounded to bf16 by the library itself (rt/sdpa.rs:167-181): with the fold switch on (opt-in) that
     one rounding is of q * scale * log2(e) and the kernel runs its form for scale = ln 2. Checked: the launch counter
     of that form moves; the result IS the kernel-level call on bf16(q * c) at ln 2, bit for bit; against the fp32
     host math on the UNROUNDED q at the plan's scale it is inside the tolerance and as close as the unfolded order
@@ -176,7 +218,7 @@ def test_f32_queries_take_the_scale_into_their_one_rounding(fv, oracle, kind):
         with fv.with_fold_scale(False):
             plain = fv.sdpa(tq, tk, tv, plan)
         assert lib.fv_sdpa_log2_domain_launches() == n0 + 1
-        assert fv.fold_scale()                                                # the default is on
+        assert not fv.fold_scale()                                            # the default is the reference's order
         # bf16 queries: the switch changes nothing
         q16 = tq.to(torch.bfloat16)
         with fv.with_fold_scale(True):

@@ -190,6 +190,39 @@ def test_fine_stage_vs_f64_block_sparse(fv, oracle, grid):
         assert np.array_equal(part.cpu().numpy(), sparse[:, 64:(nb - 1) * 64])
 
 
+def test_whole_op_folds_the_scale_into_the_one_rounding_of_f32_queries(fv, oracle):
+    """f32 q gets its one rounding to bf16 in the whole op's tile pass: with the fold switch on (opt-in) that is the
+    rounding of q * scale * log2(e), and the fine kernel runs its form without the per-score multiply. On a q that
+    is NOT made of bf16 numbers both orders are equally close to the host oracle, the selection (which never sees
+    the rounded copy) is the same list for list, and bf16 operands, which are already rounded, are left alone."""
+    import torch
+
+    grid = (5, 6, 9)
+    announce(f"vsa whole op, scale folded into f32 q, grid={grid}")
+    ctx = fv.VsaCtx(grid, 0.8)
+    oplan = oracle.TilePlan(grid)
+    q, k, v, g = vsa_inputs(oracle, 67, 2, ctx.seq)
+    q = randn(670, q.shape)                                    # f32 values off the bf16 grid
+    scale = np.float32(1.0 / np.sqrt(D))
+    want = oracle.vsa_attention_host(q, k, v, g, oplan, ctx.topk, 1, 2, D, scale)
+    args = [dev(x) for x in (q, k, v, g)]
+    assert not fv.fold_scale()                                  # the default is the reference's order
+    plain, sel_p = fv.vsa_attention_device(*args, ctx, float(scale), return_selected=True)
+    with fv.with_fold_scale(True):
+        folded, sel_f = fv.vsa_attention_device(*args, ctx, float(scale), return_selected=True)
+    torch.cuda.synchronize()
+    assert torch.equal(sel_f, sel_p) and not torch.equal(folded, plain)
+    mf = assert_parity(folded.cpu().numpy(), want, "vsa_op_f32_folded")
+    mp = assert_parity(plain.cpu().numpy(), want, "vsa_op_f32_unfolded")
+    assert mf["rel_l2"] <= 1.1 * mp["rel_l2"] and mf["rel_l2"] <= 2e-2
+    b16 = [x.to(torch.bfloat16) for x in args]
+    a = fv.vsa_attention_device(*b16, ctx, float(scale))
+    with fv.with_fold_scale(True):
+        b = fv.vsa_attention_device(*b16, ctx, float(scale))
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("grid", GRIDS)
 @pytest.mark.parametrize("in_bf16", [False, True])
 def test_whole_op_vs_host_oracle(fv, oracle, grid, in_bf16):
