@@ -69,16 +69,20 @@ def test_block_causal_matches_masked_oracle(fv, oracle, bh, s, bt, win, sink, d)
     assert_bf16_result_matches_f32_result(got16.float().cpu().numpy(), got, f"causal_{s}_{bt}_{win}_{sink}", exact_share=0.9)
 
 
-def test_one_block_spanning_the_sequence_is_the_dense_kernel(fv):
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("out_bf16", [False, True])
+def test_one_block_spanning_the_sequence_is_the_dense_kernel(fv, d, out_bf16):
+    """gpucheck/src/kernels_wan.rs:230-261 (its shape: 1 x 3 x 333, both head dims, bf16 result), and a longer one."""
     import torch
 
-    bh, s, d = 3, 700, 128
-    announce("causal one-block == dense, 3x700")
-    q, k, v = (to_dev_bf16(x) for x in qkv(11, bh, s, s, d))
-    dense = fv.sdpa_dense_bf16(q, k, v)
-    causal = fv.sdpa_block_causal_bf16(q, k, v, 4096, 0, 0)
-    torch.cuda.synchronize()
-    assert torch.equal(dense, causal)
+    for bh, s in ((3, 333), (3, 700)):
+        announce(f"causal one-block == dense, {bh}x{s} d={d} out_bf16={out_bf16}")
+        q, k, v = (to_dev_bf16(x) for x in qkv(11 + s, bh, s, s, d))
+        dense = fv.sdpa_dense_bf16(q, k, v, out_bf16=out_bf16)
+        causal = fv.sdpa_block_causal_bf16(q, k, v, max(s, 4096), 0, 0, out_bf16=out_bf16)
+        exact = fv.sdpa_block_causal_bf16(q, k, v, s, 0, 0, out_bf16=out_bf16)
+        torch.cuda.synchronize()
+        assert torch.equal(dense, causal) and torch.equal(dense, exact)
 
 
 def test_sq_ne_sk_and_first_block_rows(fv, oracle):
