@@ -45,16 +45,15 @@ int fv_sdpa_init(void);
  * 1 <= b*h <= 65535, lengths fit int32. */
 int fv_sdpa_supported(size_t b, size_t h, size_t sq, size_t sk, size_t d);
 
-/* No counterpart in the reference. The fused kernels work in base 2: P = 2^(scale * log2(e) * s - offset),
- * one multiply-add and one v_exp_f32 per score. A caller that folds its softmax scale and log2(e) into Q before
- * Q's one rounding to bf16 (for Wan: multiply the weight of the q RMSNorm, fv_qk_norm_rope_bhsd's `w`, by
- * scale * log2(e)) and passes scale = FV_SDPA_SCALE_LOG2_DOMAIN gets scale * log2(e) == 1 exactly, and every
- * fused entry (dense, strided, split-KV, block-causal, VDN window) then runs a form whose softmax offset rides
- * in the C operand of the K Q^T MFMAs and whose multiply-add per score is gone: 3.6 % faster at H=12 S=32760,
- * 8 % on block-causal launches and at head dim 64. Same arithmetic otherwise, same tolerance against the host
- * math at the same operands and scale. fv_vsa_fine (and through it fv_vsa_attention, whose coarse stage uses
- * the scale as given) takes the same form at that scale. fv_sdpa_is_log2_domain_scale: 1 when `scale` selects
- * that form. */
+/* No counterpart in the reference. The fused kernels work in base 2 with the softmax offset riding in the C
+ * operand of the K Q^T MFMAs: P = 2^(scale * log2(e) * (s - offset)), one multiply and one v_exp_f32 per score.
+ * A caller that folds its softmax scale and log2(e) into Q before Q's one rounding to bf16 (for Wan: pass
+ * out_mul = scale * log2(e) to fv_qk_norm_rope_bhsd) and passes scale = FV_SDPA_SCALE_LOG2_DOMAIN gets
+ * scale * log2(e) == 1 exactly, and every fused entry (dense, strided, split-KV, block-causal, VDN window) then
+ * runs a form without that multiply: 1.7 % faster at H=12 S=32760, more at head dim 64. Same arithmetic
+ * otherwise, same tolerance against the host math at the same operands and scale. fv_vsa_fine (and through it
+ * fv_vsa_attention, whose coarse stage uses the scale as given) takes the same form at that scale.
+ * fv_sdpa_is_log2_domain_scale: 1 when `scale` selects that form. */
 #define FV_SDPA_SCALE_LOG2_DOMAIN 0.6931471805599453f /* ln 2 */
 int fv_sdpa_is_log2_domain_scale(float scale);
 /* Launches of that form of the dense / masked kernel since the library was loaded (all its entries together). */
