@@ -170,6 +170,37 @@ def test_declines(fv):
     assert not fv.sdpa_supported(2, 40000, 64, 64, 128)
 
 
+@pytest.mark.parametrize("out_bf16", [False, True])
+def test_largest_batch_times_heads(fv, oracle, out_bf16):
+    """The reference's launch limit (rt/attn.rs:112-128: 1 <= b * h <= 65535) at its upper end: 65535 heads of a ragged
+    little call, dense and block-causal, the first and last heads and a seeded sample checked against the host math;
+    one head more declines."""
+    import torch
+
+    bh, sq, sk, d = 65535, 9, 70, 128
+    announce(f"dense + block-causal at bh={bh}, out_bf16={out_bf16}")
+    g = torch.Generator(device="cuda").manual_seed(65535)
+    q = torch.randn((bh, sq, d), generator=g, device="cuda").to(torch.bfloat16)
+    k = torch.randn((bh, sk, d), generator=g, device="cuda").to(torch.bfloat16)
+    v = torch.randn((bh, sk, d), generator=g, device="cuda").to(torch.bfloat16)
+    got = fv.sdpa_dense_bf16(q, k, v, out_bf16=out_bf16)
+    kc, vc = k[:, :sq].contiguous(), v[:, :sq].contiguous()
+    gotc = fv.sdpa_block_causal_bf16(q, kc, vc, 2, 0, 0, out_bf16=out_bf16)
+    torch.cuda.synchronize()
+    heads = sorted({0, 1, bh - 2, bh - 1, *(int(x) for x in np.random.Generator(np.random.PCG64(5)).integers(0, bh, 28))})
+    host = lambda t: t[heads].float().cpu().numpy()
+    want = oracle.sdpa_f64(host(q), host(k), host(v))
+    wantc = oracle.sdpa_f64(host(q), host(kc), host(vc), mask_bc=(2, 0, 0))
+    bar = REL_L2_BF16_OUT if out_bf16 else REL_L2_F32_OUT
+    assert_parity(host(got), want, "dense_bh65535", max_rel_l2=bar)
+    assert_parity(host(gotc), wantc, "causal_bh65535", max_rel_l2=bar)
+    assert torch.isfinite(got.float()).all() and torch.isfinite(gotc.float()).all()
+    assert fv.sdpa_supported(1, bh, sq, sk, d) and not fv.sdpa_supported(1, bh + 1, sq, sk, d)
+    one_more = torch.zeros((bh + 1, 1, d), device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(fv.FvDeclined):
+        fv.sdpa_dense_bf16(one_more, one_more, one_more)
+
+
 def test_headline_shape_sampled_rows(fv, oracle):
     """Wan-1.3B 480p self-attention at full size (S = 32760, H = 12), inputs from numpy's PCG64: parity of
     every head on more than 1024 query rows, the first and last row of several 256-query workgroup tiles
