@@ -170,6 +170,36 @@ def test_declines(fv):
     assert not fv.sdpa_supported(2, 40000, 64, 64, 128)
 
 
+@pytest.mark.parametrize("bh,s", [(2, 300), (4, 1000), (8, 4097)])
+def test_peaked_regime(fv, oracle, bh, s):
+    """The reference's `peaked` input regime (gpucheck/src/kernels_attn.rs:108-131: q scaled by 3, a per-channel offset
+    of std 2 on K, bf16-valued): rows dominated by a few keys, scores of tens of units, the regime in which the
+    softmax offset policy shows if it shows anywhere. f32 results (running max) against the f64 host math at the
+    reference's 2e-3, bf16 results (offset fixed after the first 128 keys) at its 1e-2, and no workgroup had to
+    repeat its pass."""
+    import torch
+
+    d = 128
+    announce(f"dense, peaked inputs, bh={bh} s={s}")
+    rng = np.random.Generator(np.random.PCG64(108 + s))
+    q = rng.standard_normal((bh, s, d), dtype=np.float32) * np.float32(3.0)
+    k = rng.standard_normal((bh, s, d), dtype=np.float32) + (rng.standard_normal((bh, 1, d), dtype=np.float32) * np.float32(2.0))
+    v = rng.standard_normal((bh, s, d), dtype=np.float32)
+    q, k, v = (oracle.quantize_bf16(x) for x in (q, k, v))
+    want = oracle.sdpa_f64(q, k, v)
+    tq, tk, tv = (to_dev_bf16(x) for x in (q, k, v))
+    n0 = fv.lib().fv_sdpa_exact_pass_reruns()
+    got = fv.sdpa_dense_bf16(tq, tk, tv).cpu().numpy()
+    got16 = fv.sdpa_dense_bf16(tq, tk, tv, out_bf16=True).float().cpu().numpy()
+    torch.cuda.synchronize()
+    m32, m16 = metrics(got, want), metrics(got16, want)
+    print(f"[peaked] f32 result rel_l2 {m32['rel_l2']:.3e} max_abs {m32['max_abs']:.2e}; bf16 result rel_l2 {m16['rel_l2']:.3e} "
+          f"max_abs {m16['max_abs']:.2e} (largest |out| {np.abs(want).max():.2f})", flush=True)
+    assert m32["rel_l2"] <= REL_L2_F32_OUT and m32["cosine"] >= 0.9999
+    assert m16["rel_l2"] <= REL_L2_BF16_OUT and m16["cosine"] >= 0.9999
+    assert fv.lib().fv_sdpa_exact_pass_reruns() == n0
+
+
 @pytest.mark.parametrize("out_bf16", [False, True])
 def test_largest_batch_times_heads(fv, oracle, out_bf16):
     """The reference's launch limit (rt/attn.rs:112-128: 1 <= b * h <= 65535) at its upper end: 65535 heads of a ragged
