@@ -271,6 +271,42 @@ def test_backend_setting_steers_the_dense_route(fv, oracle):
     assert fv.rt_stats()["fused"] == before["fused"] + 1
 
 
+@pytest.mark.parametrize("b,h,sq,sk,d", [(1, 4, 256, 256, 128), (1, 4, 256, 77, 128), (2, 2, 130, 130, 64), (1, 2, 96, 96, 80)])
+@pytest.mark.parametrize("act16", [False, True])
+def test_every_plan_the_families_call_runs_on_the_device(fv, oracle, b, h, sq, sk, d, act16):
+    """gpucheck/src/kernels.rs:2813-2897, as it would run against this library: every plan the model families build
+    (dense, dense with fp8_first, masked with a zero mask, both KV-window forms, block-causal and the VDN window where
+    the shape allows), f32 tensors in, f32 and bf16 activations, the fused head dims and one the fused kernels
+    decline (d = 80): each call succeeds with a device-resident result of the context's dtype; here the values are
+    checked too, against the host math under the plan's mask."""
+    import torch
+
+    announce(f"rt every plan {b}x{h}x{sq}x{sk}x{d} act16={act16}")
+    q, k, v = qkv(2813 + sq + sk + d, b * h, sq, sk, d, round_bf16=False)
+    t4 = lambda x, s: dev(x.reshape(b, h, s, d))
+    tq, tk, tv = t4(q, sq), t4(k, sk), t4(v, sk)
+    zero_mask = torch.zeros((1, 1, sq, sk), device="cuda", dtype=torch.float32)
+    plans = [("dense", fv.Plan.dense(None), None), ("dense_fp8_first", fv.Plan.dense(None).fp8_first(), None),
+             ("masked", fv.Plan.masked(None, zero_mask), None), ("kv_window", fv.Plan.kv_window(), None),
+             ("kv_window_reference", fv.Plan.kv_window_with(False), None)]
+    if sq == sk:
+        plans.append(("block_causal", fv.Plan.block_causal(None, fv.BlockCausal(64, 0, 0)),
+                      oracle.block_causal_dense_mask(64, 0, 0, sq, sk)))
+    if sq == sk and d == 128:
+        plans.append(("vdn_window", fv.Plan.vdn_window(None, fv.VdnWindow(16, 16, 15, 0, 1)),
+                      oracle.vdn_window_dense_mask(16, 16, 15, 0, 1, sq, sk)))
+    for name, plan, mask in plans:
+        with fv.with_bf16_act(act16):
+            out = fv.sdpa(tq, tk, tv, plan)
+        torch.cuda.synchronize()
+        assert out.is_cuda and tuple(out.shape) == (b, h, sq, d), name
+        assert out.dtype == (torch.bfloat16 if act16 else torch.float32), name
+        want = oracle.sdpa_composed(q, k, v, mask=mask)
+        m = metrics(out.float().cpu().numpy().reshape(b * h, sq, d), want)
+        print(f"[every plan] {name}: rel_l2 {m['rel_l2']:.3e} max_abs {m['max_abs']:.2e}", flush=True)
+        assert m["rel_l2"] <= 1e-2 and m["cosine"] >= 0.9999, (name, m)
+
+
 def test_block_causal_and_kv_window_plans_at_d128(fv, oracle):
     import torch
 
