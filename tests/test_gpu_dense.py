@@ -381,6 +381,41 @@ def test_extreme_score_ranges(fv, oracle, d):
 
 
 @pytest.mark.parametrize("d", [128, 64])
+def test_scores_that_fall_away_from_the_first_maximum(fv, oracle, d):
+    """The other direction: the first 128 keys hold the row's largest scores and everything after them lies hundreds of
+    base-2 units below (their P underflows to zero against either offset), and rows whose scores fall steadily so that
+    the weights thin out over many orders of magnitude. The fixed offset is the right one from the start: no workgroup
+    repeats its pass, bf16 and f32 results both match the f64 host math, and a growth just under the acceptance bound
+    (about 2^65 here) passes without a repeat as well."""
+    import torch
+
+    bh, sq, sk = 3, 300, 900
+    announce(f"dense fixed-offset pass, falling scores d={d}")
+    rng = np.random.Generator(np.random.PCG64(2424))
+    q = np.abs(rng.standard_normal((bh, sq, d)).astype(np.float32)) + 1.0
+    k = rng.standard_normal((bh, sk, d)).astype(np.float32) * np.float32(0.05)
+    v = oracle.quantize_bf16(rng.standard_normal((bh, sk, d)).astype(np.float32))
+    u = np.ones(d, dtype=np.float32)
+    k[0, 128:] -= 20.0 * u                                                     # head 0: a cliff after the first 128 keys
+    k[1] -= (np.linspace(0.0, 6.0, sk, dtype=np.float32)[:, None]) * u         # head 1: a steady slide
+    # head 2: growth of about 60 base-2 units past the first 128 keys, inside the bound (2^100 for the row sum)
+    k[2, 128:] += np.float32(60.0 / (1.4427 * (1.0 / np.sqrt(d)) * 1.8 * d)) * u
+    q, k = oracle.quantize_bf16(q), oracle.quantize_bf16(k)
+    tq, tk, tv = (to_dev_bf16(x) for x in (q, k, v))
+    lib = fv.lib()
+    n0 = lib.fv_sdpa_exact_pass_reruns()
+    got16 = fv.sdpa_dense_bf16(tq, tk, tv, out_bf16=True)
+    got32 = fv.sdpa_dense_bf16(tq, tk, tv)
+    torch.cuda.synchronize()
+    assert lib.fv_sdpa_exact_pass_reruns() == n0
+    want = oracle.sdpa_f64(q, k, v)
+    growth = (q[2].astype(np.float64) @ k[2].astype(np.float64).T) * (1.4427 / np.sqrt(d))
+    print(f"head 2: scores past the first 128 keys exceed the first maximum by {(growth[:, 128:].max(1) - growth[:, :128].max(1)).max():.1f} base-2 units")
+    assert_parity(got32.cpu().numpy(), want, f"dense_falling_f32_d{d}", max_rel_l2=REL_L2_F32_OUT)
+    assert_parity(got16.float().cpu().numpy(), want, f"dense_falling_bf16_d{d}", max_abs=2e-2, max_rel_l2=REL_L2_BF16_OUT)
+
+
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("out_bf16", [False, True])
 def test_scores_that_outgrow_the_first_maximum_redo_the_pass(fv, oracle, d, out_bf16):
     """Dense launches that write bf16 fix every query's softmax offset at the largest score of its first 128 keys and
